@@ -76,6 +76,8 @@ class EngineConfig:
     # GPU weight copies: "dual" (row-major for prefill + shuffled for decode), "shuffled" (shuffled
     # only; prefill unshuffles per GEMM into scratch), "auto" = dual when 2x weights <= 35% of HBM
     weight_residency: str = "auto"
+    # sequences that may be live at once on a model with a per-sequence running state (its slots)
+    state_slots: int = 16
 
 
 @dataclass
@@ -174,8 +176,12 @@ class Engine:
     def _alloc_kv(self) -> PagedKVCache:
         m = self.model
         bs = self.ecfg.block_size
-        per_block = PagedKVCache.bytes_per_block(self.cfg.n_layers, m.kv_heads_local, self.cfg.head_dim, bs,
-                                                 torch.finfo(self.dtype).bits // 8)
+        own = hasattr(m, "make_cache")      # the model brings its cache layout (latent rows + state slots)
+        if own:
+            per_block = m.cache_bytes_per_block(bs, torch.finfo(self.dtype).bits // 8)
+        else:
+            per_block = PagedKVCache.bytes_per_block(self.cfg.n_layers, m.kv_heads_local, self.cfg.head_dim, bs,
+                                                     torch.finfo(self.dtype).bits // 8)
         nb = self.ecfg.num_blocks
         if nb is None and self.ecfg.kv_budget_bytes is not None:
             nb = max(64, int(self.ecfg.kv_budget_bytes) // per_block)
@@ -194,8 +200,13 @@ class Engine:
             # them or none (a pool sized from one rank's free memory, e.g. a second rehearsal rank
             # on a shared GPU, could run out alone and skip collectives its peers enter)
             nb = self.tp.group_min(int(nb))
-        kv = PagedKVCache(self.cfg.n_layers, m.kv_heads_local, self.cfg.head_dim, int(nb), bs,
-                          self.device, self.dtype)
+        if own:
+            # one slot more than the live sequences: padded rows of a captured decode step use it
+            kv = m.make_cache(int(nb), bs, self.device, self.dtype, self.ecfg.state_slots + 1)
+            self._scratch_slot = kv.state.take()
+        else:
+            kv = PagedKVCache(self.cfg.n_layers, m.kv_heads_local, self.cfg.head_dim, int(nb), bs,
+                              self.device, self.dtype)
         kv.max_tokens = self.cfg.max_pos   # RoPE table / block-table width (_max_blocks)
         return kv
 
@@ -219,6 +230,8 @@ class Engine:
         return self._kv is not None
 
     def kv_bytes_per_token(self) -> int:
+        if hasattr(self.model, "cache_bytes_per_block"):
+            return self.model.cache_bytes_per_block(1, torch.finfo(self.dtype).bits // 8)
         return PagedKVCache.bytes_per_block(self.cfg.n_layers, self.model.kv_heads_local, self.cfg.head_dim, 1,
                                             torch.finfo(self.dtype).bits // 8)
 
@@ -412,6 +425,114 @@ class Engine:
         s.tokens.extend(ids)
         return s, st, ids
 
+    def _varlen_meta(self, spans: Sequence[Tuple[SeqState, int, Sequence[int]]], rows: Optional[List[int]] = None):
+        """Device inputs of one varlen forward over ``spans`` = (sequence, first position, ids), each
+        span's K/V slots already reserved: (token ids, positions, attention metadata). ``rows``:
+        the batch rows whose logits are wanted (default: every span's last row)."""
+        dev = self.device
+        tok, pos, slots, cu, starts, last = [], [], [], [0], [], []
+        seqs = []
+        for s, st, chunk in spans:
+            take = len(chunk)
+            tok += chunk
+            pos += list(range(st, st + take))
+            slots += self.kv.slots(s, st, st + take)
+            starts.append(st)
+            cu.append(cu[-1] + take)
+            last.append(cu[-1] - 1)
+            seqs.append(s)
+        maxb = max(len(s.blocks) for s in seqs)
+        bt = torch.zeros(len(seqs), maxb, dtype=torch.int32)
+        for j, s in enumerate(seqs):
+            bt[j, :len(s.blocks)] = torch.tensor(s.blocks, dtype=torch.int32)
+        cu_t = torch.tensor(cu, dtype=torch.int32)
+        st_t = torch.tensor(starts, dtype=torch.int32)
+        meta = AttnMeta(kind="prefill",
+                        slot_mapping=torch.tensor(slots, dtype=torch.int64).to(dev, non_blocking=True),
+                        block_tables=bt.to(dev, non_blocking=True),
+                        cu_q=cu_t.to(dev, non_blocking=True),
+                        start_pos=st_t.to(dev, non_blocking=True),
+                        last_rows=torch.tensor(last if rows is None else rows, dtype=torch.int64).to(dev, non_blocking=True))
+        if self.debug_checks:
+            self.check_paging(bt, slots)
+        if getattr(self.model, "stateful", False):
+            # the running state of every sequence follows its rows: slot per sequence, and the
+            # state then belongs to exactly the tokens fed so far
+            meta.state_slots = torch.tensor([self.kv.slot_of(s) for s in seqs], dtype=torch.int32).to(dev, non_blocking=True)
+            meta.row_seq = torch.repeat_interleave(torch.arange(len(seqs), dtype=torch.int32),
+                                                   cu_t[1:] - cu_t[:-1]).to(dev, non_blocking=True)
+            meta.host_rows = (cu_t, st_t)
+            for s, st, chunk in spans:
+                s.state_len = st + len(chunk)
+        elif self.on_gpu:
+            rows_pt = ops.native().prefill_rows_per_tile(self.model.n_heads // self.model.n_kv_heads,
+                                                         self.cfg.head_dim)
+            meta.tile_map = ops.prefill_tile_map(cu_t, rows_pt, st_t).to(dev, non_blocking=True)
+            # few tiles x KV heads (a tensor-parallel shard) leave most CUs idle: cut the long
+            # tiles' key ranges into partials merged by a second launch (attention_prefill32.hip)
+            G = self.model.n_heads // self.model.n_kv_heads
+            if self.ecfg.prefill_key_split and ops.native().prefill_split_supported(G, self.cfg.head_dim):
+                plan = ops.prefill_split_plan(cu_t, rows_pt, st_t, self.model.n_kv_heads)
+                if plan is not None:
+                    meta.prefill_split = (plan[0].to(dev, non_blocking=True), plan[1].to(dev, non_blocking=True),
+                                          plan[2])
+        return (torch.tensor(tok, dtype=torch.int64).to(dev, non_blocking=True),
+                torch.tensor(pos, dtype=torch.int64).to(dev, non_blocking=True), meta)
+
+    @torch.no_grad()
+    def step(self, entries: Sequence[Tuple[str, Sequence[int], Sequence[int]]], end: Sequence[str] = ()) -> torch.Tensor:
+        """One batched forward over the NEXT tokens of several live sequences: whole prompts,
+        portions of prompts and single decoded tokens side by side. ``entries`` = (sequence key,
+        its next token ids, the places among them whose logits are wanted); a key seen for the
+        first time is admitted (blocks and, for stateful models, a state slot). Returns the
+        wanted logits [n, vocab] fp32 in entry order. ``end``: keys whose blocks and state are
+        given back after the step. Steps made only of single tokens of running sequences take
+        the decode launch (split keys), every other step the varlen launch."""
+        with self._on_stream():
+            spans = [self.reserve(self.kv.seq(key), toks) for key, toks, _ in entries]
+            single = all(len(ids) == 1 and st > 0 for _, st, ids in spans)
+            rows, at = [], 0
+            for (_, _, ids), (_, _, want) in zip(spans, entries):
+                rows += [at + int(w) for w in want]
+                at += len(ids)
+            if single:
+                logits = self._decode_rows(spans)
+                out = logits.index_select(0, torch.tensor(rows, dtype=torch.int64, device=logits.device))
+            else:
+                tok, pos, meta = self._varlen_meta(spans, rows)
+                with trace.range("step"):
+                    out = self.model.forward(tok, pos, self.kv, meta)
+            self.stats["prefill_tokens"] += 0 if single else at
+            self.stats["decode_tokens"] += at if single else 0
+            for key in end:
+                self.release(key)
+            return out.float()
+
+    def _decode_rows(self, spans: Sequence[Tuple[SeqState, int, Sequence[int]]]) -> torch.Tensor:
+        """One eager decode-kind forward: span b feeds ONE token at position ``st`` of its sequence."""
+        dev = self.device
+        seqs = [s for s, _, _ in spans]
+        B = len(seqs)
+        pos = [st for _, st, _ in spans]
+        bt = torch.zeros(B, max(len(s.blocks) for s in seqs), dtype=torch.int32)
+        for j, s in enumerate(seqs):
+            bt[j, :len(s.blocks)] = torch.tensor(s.blocks, dtype=torch.int32)
+        slots = [self.kv.slots(s, p, p + 1)[0] for s, p in zip(seqs, pos)]
+        meta = AttnMeta(kind="decode", slot_mapping=torch.tensor(slots, dtype=torch.int64).to(dev, non_blocking=True),
+                        block_tables=bt.to(dev, non_blocking=True),
+                        ctx_lens=torch.tensor([p + 1 for p in pos], dtype=torch.int32).to(dev, non_blocking=True))
+        if getattr(self.model, "stateful", False):
+            meta.state_slots = torch.tensor([self.kv.slot_of(s) for s in seqs], dtype=torch.int32).to(dev, non_blocking=True)
+            for s, p in zip(seqs, pos):
+                s.state_len = p + 1
+        elif self.on_gpu:
+            meta.num_splits = ops.decode_splits(B, self.model.n_kv_heads)
+            meta.workspace = ops.DecodeWorkspace(B, self.model.n_heads, self.cfg.head_dim, meta.num_splits, dev)
+        if self.debug_checks:
+            self.check_paging(bt, slots)
+        ids = torch.tensor([int(ids[0]) for _, _, ids in spans], dtype=torch.int64).to(dev, non_blocking=True)
+        return self.model.forward(ids, torch.tensor(pos, dtype=torch.int64).to(dev, non_blocking=True), self.kv, meta)
+
     def prefill_reserved(self, items: Sequence[Tuple[SeqState, int, List[int]]]) -> torch.Tensor:
         """Compute the K/V of reserved spans (``reserve``) in order, chunked and varlen-batched;
         returns each span's last-token logits [S, V]."""
@@ -437,49 +558,15 @@ class Engine:
                     break
             if not batch:
                 break
-            seqs = []
-            tok, pos, slots, cu, starts, last = [], [], [], [0], [], []
+            spans = []
             for i, take in batch:
                 s, ids = pending[i]
                 st = base[i] + offs[i]
-                chunk = ids[offs[i]:offs[i] + take]
-                tok += chunk
-                pos += list(range(st, st + take))
-                slots += self.kv.slots(s, st, st + take)
-                starts.append(st)
-                cu.append(cu[-1] + take)
-                last.append(cu[-1] - 1)
+                spans.append((s, st, ids[offs[i]:offs[i] + take]))
                 offs[i] += take
-                seqs.append(s)
-            maxb = max(len(s.blocks) for s in seqs)
-            bt = torch.zeros(len(seqs), maxb, dtype=torch.int32)
-            for j, s in enumerate(seqs):
-                bt[j, :len(s.blocks)] = torch.tensor(s.blocks, dtype=torch.int32)
-            cu_t = torch.tensor(cu, dtype=torch.int32)
-            meta = AttnMeta(kind="prefill",
-                            slot_mapping=torch.tensor(slots, dtype=torch.int64).to(dev, non_blocking=True),
-                            block_tables=bt.to(dev, non_blocking=True),
-                            cu_q=cu_t.to(dev, non_blocking=True),
-                            start_pos=torch.tensor(starts, dtype=torch.int32).to(dev, non_blocking=True),
-                            last_rows=torch.tensor(last, dtype=torch.int64).to(dev, non_blocking=True))
-            if self.debug_checks:
-                self.check_paging(bt, slots)
-            if self.on_gpu:
-                rows = ops.native().prefill_rows_per_tile(self.model.n_heads // self.model.n_kv_heads,
-                                                          self.cfg.head_dim)
-                meta.tile_map = ops.prefill_tile_map(cu_t, rows, torch.tensor(starts)).to(dev, non_blocking=True)
-                # few tiles x KV heads (a tensor-parallel shard) leave most CUs idle: cut the long
-                # tiles' key ranges into partials merged by a second launch (attention_prefill32.hip)
-                G = self.model.n_heads // self.model.n_kv_heads
-                if self.ecfg.prefill_key_split and ops.native().prefill_split_supported(G, self.cfg.head_dim):
-                    plan = ops.prefill_split_plan(cu_t, rows, torch.tensor(starts), self.model.n_kv_heads)
-                    if plan is not None:
-                        meta.prefill_split = (plan[0].to(dev, non_blocking=True), plan[1].to(dev, non_blocking=True),
-                                              plan[2])
+            tok, pos, meta = self._varlen_meta(spans)
             with trace.range("prefill"):
-                logits = self.model.forward(torch.tensor(tok, dtype=torch.int64).to(dev, non_blocking=True),
-                                            torch.tensor(pos, dtype=torch.int64).to(dev, non_blocking=True),
-                                            self.kv, meta)
+                logits = self.model.forward(tok, pos, self.kv, meta)
             for j, (i, take) in enumerate(batch):
                 if offs[i] >= len(pending[i][1]):
                     last_logits[i] = logits[j]
@@ -854,6 +941,7 @@ class Engine:
                 toks = self._decode_eager(seqs, chunk, first, steps + 1, time.perf_counter() + 1e9, eos, groups)
         out = []
         for sq, tk, f in zip(seqs, toks, last):
+            sq.state_len = sq.length + len(tk) - 1 if not getattr(runner, "overshoot", 0) else -1
             new = list(tk[1:steps + 1])
             sq.tokens.extend([int(f)] + new[:-1])     # K/V now covers the old last token + all but the newest
             out.append(new)
@@ -894,6 +982,8 @@ class Engine:
         gen: List[List[int]] = []
         self._dev_gen: List[Optional[torch.Tensor]] = []
         for b, (s, t) in enumerate(zip(seqs, turns)):
+            # a running state has seen every token that was fed: all sampled ones but the newest
+            s.state_len = s.length + len(toks[b]) - 1 if not getattr(runner, "overshoot", 0) else -1
             g = toks[b][:max_new[b]]
             if not t.params.ignore_eos:
                 g = cut_at_stop(g, eos)
@@ -943,20 +1033,26 @@ class Engine:
             bt[j, :len(s.blocks)] = torch.tensor(s.blocks, dtype=torch.int32)
         bt = bt.to(dev)
         bucket = next((b for b in BATCH_BUCKETS if b >= B), B)
-        splits = ops.decode_splits(bucket, self.model.n_kv_heads, grouped=groups is not None) if self.on_gpu else 1
+        own_attn = hasattr(self.model, "make_cache")    # the model sizes its own attention launch
+        splits = (ops.decode_splits(bucket, self.model.n_kv_heads, grouped=groups is not None)
+                  if self.on_gpu and not own_attn else 1)
         G = self.model.n_heads // self.model.n_kv_heads
         ws = ops.DecodeWorkspace(B, self.model.n_heads, self.cfg.head_dim, splits, dev,
-                                 max_group=ops.MAX_GROUP_COLS // G if groups is not None else 1) if self.on_gpu else None
+                                 max_group=ops.MAX_GROUP_COLS // G if groups is not None else 1) \
+            if self.on_gpu and not own_attn else None
         gt = self.group_table(groups, B)
         gt = gt.to(dev) if gt is not None and self.on_gpu else None
         dist_greedy = self.dist_greedy(turns)
+        stateful = getattr(self.model, "stateful", False)
+        st_slots = torch.tensor([self.kv.slot_of(s) for s in seqs], dtype=torch.int32, device=dev) if stateful else None
         for step in range(1, steps):
             pos = list(lens)
             slots = [s.blocks[p // self.kv.block_size] * self.kv.block_size + p % self.kv.block_size
                      for s, p in zip(seqs, pos)]
             meta = AttnMeta(kind="decode", slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev),
                             block_tables=bt, ctx_lens=torch.tensor([p + 1 for p in pos], dtype=torch.int32, device=dev),
-                            num_splits=splits, workspace=ws, groups=gt, local_logits=dist_greedy)
+                            num_splits=splits, workspace=ws, groups=gt, local_logits=dist_greedy,
+                            state_slots=st_slots)
             logits = self.model.forward(cur.to(dev), torch.tensor(pos, dtype=torch.int64, device=dev), self.kv, meta)
             offs = torch.tensor([p + 1 for p in pos], dtype=torch.int64, device=dev)
             if dist_greedy:

@@ -81,6 +81,10 @@ class DecodeGraph:
         self.slots = torch.zeros(B, dtype=torch.int64, device=dev)
         self.offsets = torch.zeros(B, dtype=torch.int64, device=dev)
         self.hidden = torch.zeros(B, engine.model.cfg.hidden, dtype=engine.model.dtype, device=dev)
+        # models with a per-sequence running state: each row's state slot (padded rows: the scratch slot)
+        self.stateful = getattr(engine.model, "stateful", False)
+        self.state_slots = (torch.full((B,), engine._scratch_slot, dtype=torch.int32, device=dev)
+                            if self.stateful else None)
         G = engine.model.n_heads // engine.model.n_kv_heads
         self.ws = ops.DecodeWorkspace(B, engine.model.n_heads, engine.cfg.head_dim, max(1, splits), dev,
                                       max_group=ops.MAX_GROUP_COLS // G if grouped else 1)
@@ -125,7 +129,8 @@ class DecodeGraph:
             ops.paging_guard(self.block_tables, self.ctx_lens, self.positions, slots, self.guard_err,
                              e.kv.num_blocks, self.bs)
         meta = AttnMeta(kind="decode", slot_mapping=slots, block_tables=self.block_tables, ctx_lens=self.ctx_lens,
-                        num_splits=self.splits, workspace=self.ws, groups=self.groups, local_logits=self.dist_greedy)
+                        num_splits=self.splits, workspace=self.ws, groups=self.groups, local_logits=self.dist_greedy,
+                        state_slots=self.state_slots)
         if hidden is not None:
             logits = e.model.forward(self.input_ids, self.positions, e.kv, meta, hidden=hidden)
         else:
@@ -172,6 +177,8 @@ class DecodeGraph:
         self.ctx_lens.fill_(1)
         self.step.zero_()
         self.block_tables.fill_(self.scratch)
+        if self.state_slots is not None:
+            self.state_slots.fill_(self.engine._scratch_slot)
 
     def _capture(self):
         dev = self.engine.device
@@ -214,6 +221,8 @@ class DecodeGraph:
         self.block_tables.copy_(bt.to(dev, non_blocking=True))
         if self.groups is not None and groups is not None:
             self.groups.copy_(engine.group_table(groups, self.B).to(dev, non_blocking=True))
+        if self.state_slots is not None:
+            self.state_slots[:B].copy_(torch.tensor([engine.kv.slot_of(s) for s in seqs], dtype=torch.int32))
         lens = torch.tensor([s.length for s in seqs] + [0] * (self.B - B), dtype=torch.int64)
         self.positions.copy_(lens.to(dev, non_blocking=True))
         self.ctx_lens.copy_((lens + 1).to(torch.int32).to(dev, non_blocking=True))
@@ -238,6 +247,7 @@ class DecodeGraph:
         done_at = steps
         pending = None
         replays = engine.stats.get("graph_replays", 0)
+        replays0 = replays
         for i in range(1, steps):
             self.graph.replay()
             replays += 1
@@ -265,6 +275,9 @@ class DecodeGraph:
         if engine.debug_checks:
             self.check_guard()
         n = done_at - 1
+        # replays past the kept tokens: their K/V is cut off with the tokens, but a running
+        # per-sequence state has moved on with them (the engine then drops that state)
+        self.overshoot = (replays - replays0) - n
         # the same ids kept on the device, [B, n + 1] (C1 all-gathers them without host staging);
         # a copy: the next turn's replays overwrite ``out``
         self.last_dev = torch.cat([first[:B].view(1, B), self.out[:n, :B]], 0).t().contiguous()

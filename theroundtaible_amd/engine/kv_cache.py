@@ -57,6 +57,10 @@ class SeqState:
     key: str
     tokens: List[int] = field(default_factory=list)
     blocks: List[int] = field(default_factory=list)
+    # models with a running per-sequence state (input convolutions): the state slot, and how many
+    # tokens the state in it has seen (it is only valid for exactly that prefix)
+    slot: Optional[int] = None
+    state_len: int = 0
 
     @property
     def length(self) -> int:
@@ -129,17 +133,27 @@ class PagedKVCache:
 
     def truncate(self, s: SeqState, n_tokens: int) -> None:
         n_tokens = max(0, min(n_tokens, s.length))
+        n_tokens = self._state_rollback(s, n_tokens)
         keep = self.blocks_needed(n_tokens)
         for b in s.blocks[keep:]:
             self.alloc.release(b)
         del s.blocks[keep:]
         del s.tokens[n_tokens:]
 
+    def _state_rollback(self, s: SeqState, n_tokens: int) -> int:
+        """Hook of caches with a running state: the token count a roll-back to ``n_tokens`` really
+        lands on (a paged K/V cache alone can be cut anywhere)."""
+        return n_tokens
+
+    def _release_state(self, s: SeqState) -> None:
+        pass
+
     def free_seq(self, key: str) -> None:
         s = self.seqs.pop(key, None)
         if s is not None:
             for b in s.blocks:
                 self.alloc.release(b)
+            self._release_state(s)
 
     def fork(self, src: str, dst: str, copy: bool = False) -> SeqState:
         """``dst`` starts as ``src``. Default: share the blocks (refcounted prefix sharing; a writer
@@ -160,3 +174,101 @@ class PagedKVCache:
     def slots(self, s: SeqState, start: int, end: int) -> List[int]:
         bs = self.block_size
         return [s.blocks[p // bs] * bs + (p % bs) for p in range(start, end)]
+
+
+class StateSlots:
+    """Fixed pool of per-sequence state slots (the running state a model keeps beside its paged
+    cache). A slot is handed out when a sequence first runs and returned when it is freed; a
+    slot's old content is never read by its next owner (kernels treat a sequence at position 0
+    as having an all-zero state)."""
+
+    def __init__(self, n_slots: int):
+        self.n_slots = n_slots
+        self.free: List[int] = list(range(n_slots - 1, -1, -1))
+
+    def take(self) -> int:
+        if not self.free:
+            raise KVCacheOOM(f"all {self.n_slots} sequence state slots are in use")
+        return self.free.pop()
+
+    def give(self, slot: int) -> None:
+        self.free.append(slot)
+
+
+class LatentKVCache(PagedKVCache):
+    """Paged cache of latent-attention layers plus the input-convolution states.
+
+    Per layer ``l`` one tensor ``rows[l]`` ``[num_blocks, block_size, row_l]``: token ``t`` of a
+    sequence keeps ``row_l = kv_rank + rot_dim`` numbers (its normed latent, then the rotated key
+    part all heads share) at ``slot = block * block_size + offset`` — keys AND values of every
+    head are read from that one row, so a layer's cache line is 1 / (2 * heads) of a per-head
+    K/V cache's. Layers may differ in row width.
+
+    ``conv[l]`` ``[n_slots, 2, taps - 1, width]`` fp32: for each state slot the last ``taps - 1``
+    inputs of layer ``l``'s two input convolutions (mixer, feed-forward), oldest first. The state
+    belongs to exactly ``state_len`` tokens of its sequence: rolling a sequence back to any other
+    length drops it, and the sequence restarts from position 0."""
+
+    def __init__(self, row_dims, conv_width: int, taps: int, num_blocks: int, block_size: int, device,
+                 dtype=torch.bfloat16, n_slots: int = 16):
+        self.n_layers = len(row_dims)
+        self.row_dims = list(row_dims)
+        self.n_kv_heads, self.head_dim = 1, max(row_dims)
+        self.block_size, self.num_blocks = block_size, num_blocks
+        self.device, self.dtype = device, dtype
+        # zero-init: tail rows of a partial block are masked, never skipped, so they must be finite
+        self.rows = [torch.zeros(num_blocks, block_size, r, dtype=dtype, device=device) for r in row_dims]
+        self.alloc = BlockAllocator(num_blocks)
+        self.seqs = {}
+        self.taps = taps
+        self.state = StateSlots(n_slots)
+        self.conv = [torch.zeros(n_slots, 2, max(taps - 1, 1), conv_width, dtype=torch.float32, device=device)
+                     for _ in row_dims]
+
+    @staticmethod
+    def bytes_per_block(row_dims, block_size, dtype_bytes=2) -> int:   # type: ignore[override]
+        return sum(row_dims) * block_size * dtype_bytes
+
+    def layer_rows(self, l: int) -> torch.Tensor:
+        return self.rows[l]
+
+    def k_layer(self, l: int):      # the per-head views of a K/V cache do not exist here
+        raise AttributeError("a latent cache has no per-head K blocks; use layer_rows()")
+
+    v_layer = k_layer
+
+    def copy_blocks(self, src: List[int], dst: List[int]) -> None:
+        si = torch.tensor(src, dtype=torch.int64, device=self.device)
+        di = torch.tensor(dst, dtype=torch.int64, device=self.device)
+        for r in self.rows:
+            r.index_copy_(0, di, r.index_select(0, si))
+
+    def slot_of(self, s: SeqState) -> int:
+        """The sequence's state slot (taken on first use)."""
+        if s.slot is None:
+            s.slot = self.state.take()
+            s.state_len = 0
+        return s.slot
+
+    def _state_rollback(self, s: SeqState, n_tokens: int) -> int:
+        if n_tokens == s.state_len or s.slot is None:
+            return n_tokens
+        s.state_len = 0         # the convolution inputs ahead of `n_tokens` are gone: start over
+        return 0
+
+    def _release_state(self, s: SeqState) -> None:
+        if s.slot is not None:
+            self.state.give(s.slot)
+            s.slot = None
+
+    def fork(self, src: str, dst: str, copy: bool = False) -> SeqState:
+        b = super().fork(src, dst, copy=copy)
+        a = self.seqs[src]
+        if a.slot is not None and a.state_len == a.length:
+            b.slot = self.state.take()
+            b.state_len = a.state_len
+            for c in self.conv:
+                c[b.slot].copy_(c[a.slot])
+        else:
+            self.truncate(b, 0)
+        return b

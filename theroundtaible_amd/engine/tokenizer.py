@@ -36,6 +36,9 @@ class EngineTokenizer:
         self.model_vocab = model_vocab
         self.bos_id = self._tok.token_to_id("<|begin_of_text|>")
         self.eos_id = self._tok.token_to_id("<|end_of_text|>")
+        if model_vocab < self.base_vocab:   # a model smaller than the BPE: ids fold into its vocabulary
+            self.bos_id %= model_vocab
+            self.eos_id %= model_vocab
         # tokenizer family id: token-id sharing across knights requires the same (name, vocab)
         self.family = f"{self.name}/{model_vocab}"
 

@@ -86,5 +86,8 @@ class GPT2Model:
 def build_model(cfg: ModelConfig, weights, device, dtype=torch.bfloat16, tp: Optional[TPInfo] = None):
     if cfg.arch == "gpt2":
         return GPT2Model(cfg, weights, device, dtype, tp)
+    if cfg.arch == "mupulorn":
+        from .mupulorn import MupulornModel
+        return MupulornModel(cfg, weights, device, dtype, tp)
     from .llama import LlamaModel
     return LlamaModel(cfg, weights, device, dtype, tp)

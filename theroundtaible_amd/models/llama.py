@@ -45,6 +45,13 @@ class AttnMeta:
     groups: Optional[torch.Tensor] = None       # decode: [B, 3] shared-prefix groups (ops.decode_groups)
     local_logits: bool = False                  # TP decode: return this rank's vocab shard (C3 greedy argmax)
     planned: bool = False                       # decode: the workspace holds this step's ops.attn_plan
+    # models with a per-sequence running state (models/mupulorn.py): the state slot of every
+    # sequence [S] int32; varlen steps also carry each row's sequence index [T] int32, host copies
+    # of (cu_q, start_pos) for work lists built per layer shape, and those lists once built
+    state_slots: Optional[torch.Tensor] = None
+    row_seq: Optional[torch.Tensor] = None
+    host_rows: Optional[tuple] = None
+    latent_tiles: Optional[dict] = None
 
 
 class LlamaModel:

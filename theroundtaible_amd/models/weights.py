@@ -72,7 +72,45 @@ def gpt2_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Optio
     return lay
 
 
+def mupulorn_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]]:
+    """Checkpoint names and shapes of a Mupulorn model (linear weights [out, in]); layers that run
+    another layer's weights have no tensors. Not tensor-parallel: every kind is None."""
+    W = cfg.hidden
+    lay: Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]] = {
+        "embed": ((cfg.vocab, W), "normal", None),
+        "final.norm": ((), "ones", None),
+        "head": ((cfg.vocab, W), "normal", None),
+    }
+    for i, ls in enumerate(cfg.layers):
+        if ls.source != i:
+            continue
+        p, m = f"l{i}.", ls.mixer
+        for n in ("norm1", "norm1b"):
+            lay[p + n] = ((), "ones", None)
+        lay[p + "canon1"] = ((W, cfg.canon_taps), "small", None)
+        lay[p + "mix.dq"] = ((m.q_rank, W), "normal", None)
+        lay[p + "mix.dq.norm"] = ((m.q_rank,), "ones", None)
+        lay[p + "mix.uq"] = ((m.heads * (m.dim + m.rot_dim), m.q_rank), "normal", None)
+        lay[p + "mix.dkv"] = ((m.kv_rank + m.rot_dim, W), "normal", None)
+        lay[p + "mix.dkv.norm"] = ((m.kv_rank,), "ones", None)
+        lay[p + "mix.uk"] = ((m.heads * m.dim, m.kv_rank), "normal", None)
+        lay[p + "mix.uv"] = ((m.heads * m.vdim, m.kv_rank), "normal", None)
+        lay[p + "mix.sink"] = ((m.heads,), "zeros", None)
+        lay[p + "mix.g"] = ((m.heads * m.vdim, W), "normal", None)
+        lay[p + "mix.o"] = ((W, m.heads * m.vdim), "normal", None)
+        if ls.ff:
+            for n in ("norm2", "norm2b"):
+                lay[p + n] = ((), "ones", None)
+            lay[p + "canon2"] = ((W, cfg.canon_taps), "small", None)
+            lay[p + "mlp.up"] = ((ls.ff, W), "normal", None)
+            lay[p + "mlp.down"] = ((W, ls.ff), "normal", None)
+            lay[p + "mlp.act"] = ((4,), "poly", None)
+    return lay
+
+
 def layout_for(cfg: ModelConfig):
+    if cfg.arch == "mupulorn":
+        return mupulorn_layout(cfg)
     return gpt2_layout(cfg) if cfg.arch == "gpt2" else llama_layout(cfg)
 
 
@@ -152,6 +190,12 @@ def _init(shape, init, std, g, device, dtype):
         return torch.ones(shape, device=device, dtype=dtype)
     if init == "zeros":
         return torch.zeros(shape, device=device, dtype=dtype)
+    if init == "poly":      # PolyNorm coefficients: equal thirds, no offset
+        return torch.tensor([1 / 3, 1 / 3, 1 / 3, 0.0], device=device, dtype=dtype)
+    if init == "small":     # input-convolution taps
+        w = torch.empty(shape, device=device, dtype=dtype)
+        w.normal_(0.0, 0.1, generator=g)
+        return w
     w = torch.empty(shape, device=device, dtype=dtype)
     w.normal_(0.0, std, generator=g)
     return w
@@ -216,9 +260,21 @@ def load_safetensors(cfg: ModelConfig, path: str, device, dtype, tp: TPInfo) -> 
     tensors: Dict[str, torch.Tensor] = {}
     for f in files:
         tensors.update(load_file(f, device="cpu"))
-    name_map = _hf_gpt2_name_map(cfg) if cfg.arch == "gpt2" else _hf_llama_name_map(cfg)
     lay = layout_for(cfg)
     out = {}
+    if cfg.arch == "mupulorn":
+        # the checkpoint's own names; integer tables keep their type, everything else takes `dtype`
+        if tp.size > 1:
+            raise ValueError("mupulorn checkpoints are not tensor-parallel")
+        for name, (shape, _, _) in lay.items():
+            if name not in tensors:
+                raise KeyError(f"{path}: tensor '{name}' is missing")
+            w = tensors[name]
+            if tuple(w.shape) != tuple(shape):
+                raise ValueError(f"{path}: tensor '{name}' has shape {tuple(w.shape)}, config.json gives {tuple(shape)}")
+            out[name] = (w if not w.is_floating_point() else w.to(dtype)).to(device).contiguous()
+        return out
+    name_map = _hf_gpt2_name_map(cfg) if cfg.arch == "gpt2" else _hf_llama_name_map(cfg)
     for name, fn in name_map.items():
         if name == "lm_head" and cfg.tie_embeddings and cfg.arch == "gpt2":
             continue   # GPT-2 reads the tied head from wte; Llama-family models get a (sharded) copy

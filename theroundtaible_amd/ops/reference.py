@@ -405,3 +405,147 @@ def paging_guard(block_tables, ctx_lens, positions, slots, err, num_blocks, bloc
                 if int(slots[b]) != want:
                     code |= 4
     err[0] = int(err[0]) | code
+
+
+# ---- latent attention / input convolution / PolyNorm family (csrc/latent/*.hip) -----------------
+# Row metadata shared by these ops: ``row_seq`` [T] int32 = sequence index of every row,
+# ``positions`` [T] = absolute position of every row, ``start_pos`` [S] = position of each
+# sequence's first row in this batch (rows of a sequence are consecutive, ``cu_q`` [S + 1]).
+
+def scalar_rms_norm(x: torch.Tensor, g: torch.Tensor, eps: float, out_dtype=None) -> torch.Tensor:
+    """RMS norm whose learned weight is ONE number; fp32 math."""
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def scalar_norm_add_(res: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float) -> torch.Tensor:
+    """res (fp32, in place) += scalar_rms_norm(y, g)."""
+    res.add_(scalar_rms_norm(y, g, eps, torch.float32))
+    return res
+
+
+def canon_norm(x, g, eps, w, state, row_seq, positions, start_pos, slots, out_dtype):
+    """h + causal depthwise conv(h) with h = scalar_rms_norm(x, g): ``w`` [W, taps] (last tap =
+    the current token); inputs ahead of a sequence's first row come from ``state``
+    [n_slots, taps - 1, W] (oldest first), inputs ahead of position 0 are zero."""
+    h = scalar_rms_norm(x, g, eps, torch.float32)
+    taps = w.shape[1]
+    wf = w.float()
+    out = h * (1.0 + wf[:, taps - 1])
+    rs, pos = row_seq.long(), positions.long()
+    local = pos - start_pos.long()[rs]
+    rows = torch.arange(x.shape[0], device=x.device)
+    for k in range(1, taps):
+        in_batch = local >= k
+        src = torch.where(in_batch.unsqueeze(1), h[(rows - k).clamp(min=0)],
+                          state[slots.long()[rs], (taps - 1 - k + local).clamp(0, max(taps - 2, 0))])
+        src = torch.where((pos >= k).unsqueeze(1), src, torch.zeros_like(src))
+        out = out + wf[:, taps - 1 - k] * src
+    return out.to(out_dtype)
+
+
+def canon_state_update(x, g, eps, state, cu_q, start_pos, slots):
+    """Shift each sequence's convolution state by its rows of this batch: afterwards it holds the
+    last ``taps - 1`` normed inputs up to the sequence's newest row."""
+    keep = state.shape[1]
+    h = scalar_rms_norm(x, g, eps, torch.float32)
+    cq, sp, sl = cu_q.tolist(), start_pos.tolist(), slots.tolist()
+    for s in range(len(sl)):
+        n = cq[s + 1] - cq[s]
+        if n <= 0:
+            continue
+        old = state[sl[s]].clone()
+        for i in range(keep):
+            idx = n - keep + i              # row of this batch (>= 0) or of the old state (< 0)
+            if idx >= 0:
+                state[sl[s], i] = h[cq[s] + idx]
+            elif sp[s] + idx >= 0:
+                state[sl[s], i] = old[keep + idx]
+            else:
+                state[sl[s], i] = 0
+
+
+def rotate_interleaved(v: torch.Tensor, positions: torch.Tensor, base: float, dims: int) -> torch.Tensor:
+    """Rotary embedding on the pairs (2i, 2i + 1), i < dims / 2, of the last axis; ``v`` [T, ..., D],
+    angle = position * base^(-2i / dims) in fp32."""
+    if dims == 0:
+        return v.float()
+    i = torch.arange(dims // 2, dtype=torch.float32, device=v.device)
+    f = torch.exp2(i * (-2.0 * math.log2(base) / dims))
+    a = positions.float().view(-1, *([1] * (v.dim() - 1))) * f
+    c, s = torch.cos(a), torch.sin(a)
+    vf = v.float()
+    u, w = vf[..., 0:dims:2], vf[..., 1:dims:2]
+    out = vf.clone()
+    out[..., 0:dims:2] = u * c - w * s
+    out[..., 1:dims:2] = w * c + u * s
+    return out
+
+
+def latent_prep(proj, q_rank, kv_rank, rot_dim, wq, wkv, eps, positions, rot_base, rot_dims, cache_rows,
+                slot_mapping, out_dtype):
+    """From the fused input projection ``proj`` [T, >= q_rank + kv_rank + rot_dim]: the normed
+    query latent (returned) and the cache row (normed latent | rotated shared key part), written
+    at ``slot_mapping`` into ``cache_rows`` [num_blocks, block_size, kv_rank + rot_dim]."""
+    cq = rms_norm(proj[:, :q_rank].float(), wq.float(), eps).to(out_dtype)
+    c = rms_norm(proj[:, q_rank:q_rank + kv_rank].float(), wkv.float(), eps)
+    kr = rotate_interleaved(proj[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim], positions, rot_base, rot_dims)
+    flat = cache_rows.view(-1, cache_rows.shape[-1])
+    flat[slot_mapping.long()] = torch.cat([c, kr], -1).to(cache_rows.dtype)
+    return cq
+
+
+def latent_attention(q_lat, q, rot_off, cache_rows, block_tables, cu_q, start_pos, sink, scale, rot_base,
+                     rot_dims, out_dtype):
+    """Causal attention over the cached rows with the query folded into the latent space.
+
+    ``q_lat`` [H, T, C] (the unrotated query of each head times its key up-projection), ``q``
+    [T, H, Dq] whose entries ``rot_off:`` are the un-rotated rotary part (rotated here, by the
+    row's position). Key t = cached row, value t = its first C entries. The softmax denominator
+    also holds exp(sink_h). Returns [H, T, C]."""
+    H, T, C = q_lat.shape
+    out = torch.zeros(H, T, C, dtype=torch.float32, device=q.device)
+    cq, sp = cu_q.tolist(), start_pos.tolist()
+    BS = cache_rows.shape[1]
+    for s in range(len(sp)):
+        r0, r1 = cq[s], cq[s + 1]
+        if r1 <= r0:
+            continue
+        n = sp[s] + (r1 - r0)
+        nb = (n + BS - 1) // BS
+        K = cache_rows[block_tables[s, :nb].long()].reshape(nb * BS, -1)[:n].float()
+        pos = torch.arange(sp[s], n, device=q.device)
+        qr = rotate_interleaved(q[r0:r1, :, rot_off:], pos, rot_base, rot_dims)          # [n_q, H, R]
+        Q = torch.cat([q_lat[:, r0:r1].float(), qr.transpose(0, 1)], -1)                 # [H, n_q, C + R]
+        sc = torch.einsum("hqd,kd->hqk", Q, K) * scale
+        mask = torch.arange(n, device=q.device).view(1, 1, n) > pos.view(1, -1, 1)
+        sc = sc.masked_fill(mask, float("-inf"))
+        sk = sink.float().view(H, 1, 1)
+        m = torch.maximum(sc.max(-1, keepdim=True).values, sk)
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True) + torch.exp(sk - m)
+        out[:, r0:r1] = torch.einsum("hqk,kc->hqc", e / den, K[:, :C])
+    return out.to(out_dtype)
+
+
+def gate_mul(o, proj, g_off, out_dtype):
+    """``o`` [H, T, Dv] head-major -> [T, H * Dv], times sigmoid of ``proj[:, g_off : g_off + H * Dv]``."""
+    H, T, Dv = o.shape
+    gate = torch.sigmoid(proj[:, g_off:g_off + H * Dv].float())
+    return (o.float().permute(1, 0, 2).reshape(T, H * Dv) * gate).to(out_dtype)
+
+
+def poly_norm(z, coef, eps, out_dtype):
+    """a N(z) + b N(z^2) + c N(z^3) + e, N = divide a row by its root mean square; fp32 math."""
+    zf = z.float()
+    cf = coef.float()
+
+    def n(u):
+        return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    return (cf[0] * n(zf) + cf[1] * n(zf * zf) + cf[2] * n(zf * zf * zf) + cf[3]).to(out_dtype)
+
+
+def logit_softcap(logits, scale, cap):
+    y = logits.float() * scale
+    return cap * torch.tanh(y / cap) if cap > 0 else y
