@@ -53,7 +53,51 @@ def _run(cmd):
     return r.stderr
 
 
+def latent_ext_path() -> str:
+    return os.path.join(PKG, "_C_latent" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_latent(verbose: bool = False, jobs: int = 8) -> str:
+    """The latent-attention family's extension ``theroundtaible_amd/_C_latent*.so`` from
+    ``csrc/latent/`` — a module of its own, so a checkout that only serves such a model compiles
+    three files. Same flags as :func:`build`, plus no packed-fp32 instruction selection."""
+    src_dir = os.path.join(HERE, "latent")
+    bdir = os.path.join(BUILD, "latent")
+    os.makedirs(bdir, exist_ok=True)
+    incs, torch_lib, abi = torch_paths()
+    py_inc = sysconfig.get_paths()["include"]
+    headers = glob.glob(os.path.join(HERE, "*.h"))
+    common = ["-O3", "-fPIC", "-std=c++17", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1",
+              "-DUSE_ROCM=1", "-Wno-unused-result", "-Wno-deprecated-declarations", "-Wno-unused-command-line-argument"]
+    jobs_list, objs = [], []
+    for src in sorted(glob.glob(os.path.join(src_dir, "*.hip"))):
+        obj = os.path.join(bdir, os.path.basename(src) + ".o")
+        objs.append(obj)
+        if _newer(src, obj, headers):
+            jobs_list.append([HIPCC, "-x", "hip", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
+                              "-packed-fp32-ops", *common, "-I", HERE, "-c", src, "-o", obj])
+    bsrc = os.path.join(src_dir, "latent_bindings.cpp")
+    bobj = os.path.join(bdir, "latent_bindings.cpp.o")
+    objs.append(bobj)
+    if _newer(bsrc, bobj, []):
+        jobs_list.append([HIPCC, *common, "-I", py_inc, *sum((["-I", i] for i in incs), []),
+                          "-DTORCH_EXTENSION_NAME=_C_latent", "-DTORCH_API_INCLUDE_EXTENSION_H", "-c", bsrc, "-o", bobj])
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for err in ex.map(_run, jobs_list):
+            if verbose and err.strip():
+                print(err)
+    out = latent_ext_path()
+    if jobs_list or not os.path.exists(out):
+        tmp = out + f".{os.getpid()}.tmp"
+        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp, f"-L{torch_lib}",
+              "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lamdhip64",
+              f"-Wl,-rpath,{torch_lib}"])
+        os.replace(tmp, out)
+    return out
+
+
 def build(verbose: bool = False, jobs: int = 8) -> str:
+    build_latent(verbose, jobs)
     os.makedirs(BUILD, exist_ok=True)
     incs, torch_lib, abi = torch_paths()
     py_inc = sysconfig.get_paths()["include"]
@@ -88,4 +132,8 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    if "latent" in sys.argv[1:]:
+        print(build_latent(verbose="-v" in sys.argv))
+    else:
+        print(build(verbose="-v" in sys.argv))
+        print(latent_ext_path())

@@ -1,0 +1,310 @@
+// L3: causal attention over the paged latent cache with a softmax sink, for any head count and
+// any latent / rotary width (fp32 FMA; the cache and queries are bf16 or fp32 as templated).
+//
+// The query of every head has been folded into latent space (q_lat = q_unrotated . W_uk), so the
+// key of token t is its cached row [latent C | rotated key part R] and its value is the row's
+// first C entries: ALL heads read the SAME rows. One workgroup (4 waves) takes a tile of query
+// rows of one sequence with all their heads ("pairs" = rows x heads, PW per wave) and walks the
+// sequence's keys 64 at a time:
+//
+//   stage   the 64 cached rows (paged: block table lookup per key) into LDS, once for all pairs
+//   scores  lane = key: s[p] = sum_d q[p][d] * K[key][d]   (q in LDS, read as a broadcast)
+//   softmax online per pair (running max m, sum l), masked by each row's own position
+//   values  lane = latent column: o[p][c] += sum_key p[key] * K[key][c]   (P via LDS)
+//
+// The sink enters once, at the end: the denominator gains exp(sink_h - m). With `num_splits` > 1
+// (one query row per sequence: the decode step) a workgroup takes one contiguous range of each
+// tile's keys and writes (o, m, l) partials that `latent_combine_kernel` merges; the ranges
+// follow from the run-time position, so one captured launch serves every length.
+//
+// The rotary part of q is rotated here, on load, by the row's position (fp32 angles).
+#include "../common.h"
+
+namespace {
+
+using rt::DT;
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int KT = 64;  // keys per tile: one per lane
+
+struct AttnArgs {
+  void* out;            // [H, T, C]
+  const void* q_lat;    // [H, T, C]
+  const void* q;        // [T, H, Dq]; entries rot_off.. of a head are its rotary part
+  const void* cache;    // [num_blocks, BS, Dk], Dk = C + R
+  const int* block_tables;
+  const int* cu_q;
+  const int* start_pos;
+  const int* tiles;     // [n_tiles, 2] (sequence, first row)
+  const float* sink;    // [H]
+  float* part_o;        // [T, H, splits, C]
+  float* part_ml;       // [T, H, splits, 2]
+  int T, H, C, R, Dq, rot_off, BS, max_blocks, rows, num_splits, kstride, rot_dims;
+  int hwin;             // heads one workgroup takes (grid.z walks the windows)
+  float scale, rot_k;
+};
+
+// CPL: latent columns per lane (C <= 64 * CPL); PW: (row, head) pairs per wave
+template <typename CT, typename QT, int CPL, int PW>
+__global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int Dk = a.C + a.R;
+  CT* Ks = reinterpret_cast<CT*>(smem);                                   // [KT][kstride]
+  float* Qs = reinterpret_cast<float*>(smem + (size_t)KT * a.kstride * sizeof(CT));  // [pairs][Dk]
+  float* Ps = Qs + (size_t)kWaves * PW * Dk;                              // [pairs][KT]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int seq = a.tiles[blockIdx.x * 2], row0 = a.tiles[blockIdx.x * 2 + 1];
+  const int nrows = min(a.rows, a.cu_q[seq + 1] - row0);
+  const int pos0 = a.start_pos[seq] + (row0 - a.cu_q[seq]);   // position of the tile's first row
+  const int h0 = blockIdx.z * a.hwin;
+  const int HW = min(a.hwin, a.H - h0);     // heads of this workgroup's window
+  const int npairs = nrows * HW;
+  // this wave's pairs: p = wave * PW + i -> (row p / HW, head h0 + p % HW)
+  // ---- queries -> LDS (scaled; rotary part rotated by the row's position) ----
+  for (int p = wave; p < kWaves * PW; p += kWaves) {
+    float* qd = Qs + (size_t)p * Dk;
+    if (p >= npairs) {
+      for (int d = lane; d < Dk; d += 64) qd[d] = 0.f;
+      continue;
+    }
+    const int r = p / HW, h = h0 + p - r * HW;
+    const QT* ql = reinterpret_cast<const QT*>(a.q_lat) + ((size_t)h * a.T + row0 + r) * a.C;
+    for (int d = lane; d < a.C; d += 64) qd[d] = DT<QT>::load(ql + d) * a.scale;
+    const QT* qr = reinterpret_cast<const QT*>(a.q) + ((size_t)(row0 + r) * a.H + h) * a.Dq + a.rot_off;
+    const float posf = (float)(pos0 + r);
+    for (int i = lane; i < (a.R + 1) / 2; i += 64) {
+      const float u = DT<QT>::load(qr + 2 * i);
+      if (2 * i + 1 >= a.R) {
+        qd[a.C + 2 * i] = u * a.scale;
+        continue;
+      }
+      const float v = DT<QT>::load(qr + 2 * i + 1);
+      float cs = 1.f, sn = 0.f;
+      if (2 * i < a.rot_dims) sincosf(posf * exp2f((float)i * a.rot_k), &sn, &cs);
+      qd[a.C + 2 * i] = (u * cs - v * sn) * a.scale;
+      qd[a.C + 2 * i + 1] = (v * cs + u * sn) * a.scale;
+    }
+  }
+  float m[PW], l[PW], o[PW][CPL];
+  int qpos[PW];
+#pragma unroll
+  for (int i = 0; i < PW; ++i) {
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+    const int p = wave * PW + i;
+    qpos[i] = p < npairs ? pos0 + p / HW : -1;   // -1: no key is visible, the pair stays empty
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) o[i][j] = 0.f;
+  }
+  // ---- key range of this workgroup ----
+  const int nkeys = pos0 + nrows;   // keys 0 .. last row's position
+  int kb = 0, ke = nkeys;
+  if (a.num_splits > 1) {
+    const int ntile = (nkeys + KT - 1) / KT;
+    const int per = (ntile + a.num_splits - 1) / a.num_splits;
+    kb = min(nkeys, (int)blockIdx.y * per * KT);
+    ke = min(nkeys, kb + per * KT);
+  }
+  const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
+  const CT* cache = reinterpret_cast<const CT*>(a.cache);
+  for (int k0 = kb; k0 < ke; k0 += KT) {
+    __syncthreads();   // the previous tile's readers are done (and Qs is written, first time)
+    // stage: wave w copies keys w, w + 4, ...; lanes stride over the row
+    for (int kk = wave; kk < KT; kk += kWaves) {
+      const int kp = k0 + kk;
+      CT* dst = Ks + (size_t)kk * a.kstride;
+      if (kp < ke) {
+        const CT* src = cache + ((size_t)bt[kp / a.BS] * a.BS + kp % a.BS) * Dk;
+        for (int d = lane; d < Dk; d += 64) dst[d] = src[d];
+      } else {
+        for (int d = lane; d < Dk; d += 64) dst[d] = CT(0);
+      }
+    }
+    __syncthreads();
+    // scores: lane = key
+    float s[PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) s[i] = 0.f;
+    const CT* krow = Ks + (size_t)lane * a.kstride;
+    const float* qw = Qs + (size_t)wave * PW * Dk;
+    for (int d = 0; d < Dk; ++d) {
+      const float kv = DT<CT>::load(krow + d);
+#pragma unroll
+      for (int i = 0; i < PW; ++i) s[i] += qw[(size_t)i * Dk + d] * kv;
+    }
+    const int kp = k0 + lane;
+    float* pw = Ps + (size_t)wave * PW * KT;
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+      const bool vis = kp < ke && kp <= qpos[i];
+      const float sv = vis ? s[i] : -INFINITY;
+      const float mn = fmaxf(m[i], rt::wave_max(sv));
+      float p = 0.f, alpha = 1.f;
+      if (mn > -INFINITY) {
+        p = vis ? __expf(sv - mn) : 0.f;
+        alpha = __expf(m[i] - mn);   // m = -inf -> 0
+      }
+      l[i] = l[i] * alpha + rt::wave_sum(p);
+      m[i] = mn;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) o[i][j] *= alpha;
+      pw[i * KT + lane] = p;
+    }
+    // values: lane = latent column(s); P is read back as a broadcast (same wave wrote it)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int kk = 0; kk < KT; ++kk) {
+      float kvv[CPL];
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        const int c = lane + 64 * j;
+        kvv[j] = c < a.C ? DT<CT>::load(Ks + (size_t)kk * a.kstride + c) : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < PW; ++i) {
+        const float p = pw[i * KT + kk];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) o[i][j] += p * kvv[j];
+      }
+    }
+  }
+  // ---- finish: the sink joins the denominator (single launch) or partials go to the combine ----
+#pragma unroll
+  for (int i = 0; i < PW; ++i) {
+    const int p = wave * PW + i;
+    if (p >= npairs) continue;
+    const int r = p / HW, h = h0 + p - r * HW;
+    const int t = row0 + r;
+    if (a.num_splits > 1) {
+      float* po = a.part_o + (((size_t)t * a.H + h) * a.num_splits + blockIdx.y) * a.C;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        const int c = lane + 64 * j;
+        if (c < a.C) po[c] = o[i][j];
+      }
+      if (lane == 0) {
+        float* ml = a.part_ml + (((size_t)t * a.H + h) * a.num_splits + blockIdx.y) * 2;
+        ml[0] = m[i];
+        ml[1] = l[i];
+      }
+    } else {
+      const float sk = a.sink[h];
+      const float M = fmaxf(m[i], sk);
+      const float w = __expf(m[i] - M);
+      const float inv = 1.f / (l[i] * w + __expf(sk - M));
+      CT* orow = reinterpret_cast<CT*>(a.out) + ((size_t)h * a.T + t) * a.C;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        const int c = lane + 64 * j;
+        if (c < a.C) DT<CT>::store(orow + c, o[i][j] * w * inv);
+      }
+    }
+  }
+}
+
+// one wave per (row, head): merge the split partials and the sink
+template <typename OT>
+__global__ void __launch_bounds__(64) latent_combine_kernel(OT* __restrict__ out, const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml,
+                                                            const float* __restrict__ sink, int T, int H, int C,
+                                                            int splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* ml = part_ml + ((size_t)t * H + h) * splits * 2;
+  const float sk = sink[h];
+  float M = sk;
+  for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[2 * s]);
+  float den = __expf(sk - M);
+  for (int s = 0; s < splits; ++s) den += ml[2 * s + 1] * __expf(ml[2 * s] - M);   // l = 0 where m = -inf
+  const float inv = 1.f / den;
+  const float* po = part_o + ((size_t)t * H + h) * splits * C;
+  OT* orow = out + ((size_t)h * T + t) * C;
+  for (int c = lane; c < C; c += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float w = __expf(ml[2 * s] - M);
+      if (w > 0.f) acc += po[(size_t)s * C + c] * w;
+    }
+    DT<OT>::store(orow + c, acc * inv);
+  }
+}
+
+template <typename CT, int CPL, int PW>
+int launch_one(const AttnArgs& a, int n_tiles, size_t smem, hipStream_t stream) {
+  auto kern = latent_attn_kernel<CT, CT, CPL, PW>;
+  if (smem > 64 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      return 3;
+  }
+  hipLaunchKernelGGL(kern, dim3(n_tiles, a.num_splits, (a.H + a.hwin - 1) / a.hwin), dim3(kThreads), smem, stream, a);
+  return 0;
+}
+
+}  // namespace
+
+static int lds_stride(int Dk, size_t esz) {
+  // LDS row stride: an odd number of 4-byte words, so lane = key reads hit 64 different banks
+  int words = (int)((Dk * esz + 3) / 4);
+  if (!(words & 1)) words += 1;
+  return (int)(words * 4 / esz);
+}
+
+static size_t lds_bytes(int Dk, size_t esz, int PW) {
+  return (size_t)KT * lds_stride(Dk, esz) * esz + (size_t)kWaves * PW * Dk * 4 + (size_t)kWaves * PW * KT * 4;
+}
+
+// (row, head) pairs per wave: 8 when the staged tile, the queries and the weights fit the 160 KB
+// of LDS, else 2; 0: the row is too wide for this kernel
+static int pairs_per_wave(int Dk, bool bf) {
+  const size_t esz = bf ? 2 : 4, cap = 160 * 1024;
+  return lds_bytes(Dk, esz, 8) <= cap ? 8 : lds_bytes(Dk, esz, 2) <= cap ? 2 : 0;
+}
+
+// query rows per workgroup: all heads of a row (up to the workgroup's pairs) share the key tile
+int latent_rows_per_tile(int H, int C, int R, bool bf) {
+  const int pairs = kWaves * pairs_per_wave(C + R, bf);
+  if (pairs == 0) return 0;
+  return H >= pairs ? 1 : pairs / H;
+}
+
+// 0 ok; 1: `rows` is not latent_rows_per_tile; 2: C too wide; 3: the rows do not fit the LDS
+int launch_latent_attention(void* out, const void* q_lat, const void* q, const void* cache, const int* block_tables,
+                            const int* cu_q, const int* start_pos, const int* tiles, int n_tiles, const float* sink,
+                            float* part_o, float* part_ml, int T, int H, int C, int R, int Dq, int rot_off, int BS,
+                            int max_blocks, int rows, int num_splits, float scale, float rot_base, int rot_dims,
+                            bool bf, hipStream_t stream) {
+  if (n_tiles <= 0 || T <= 0) return 0;
+  if (C > 512) return 2;
+  const int Dk = C + R;
+  const int PW = pairs_per_wave(Dk, bf);
+  if (PW == 0) return 3;
+  const int pairs = kWaves * PW;
+  AttnArgs a;
+  a.out = out; a.q_lat = q_lat; a.q = q; a.cache = cache; a.block_tables = block_tables; a.cu_q = cu_q;
+  a.start_pos = start_pos; a.tiles = tiles; a.sink = sink; a.part_o = part_o; a.part_ml = part_ml;
+  a.T = T; a.H = H; a.C = C; a.R = R; a.Dq = Dq; a.rot_off = rot_off; a.BS = BS; a.max_blocks = max_blocks;
+  a.rows = rows; a.num_splits = num_splits; a.rot_dims = rot_dims; a.scale = scale;
+  a.rot_k = rot_dims > 0 ? (float)(-2.0 * log2((double)rot_base) / rot_dims) : 0.f;
+  a.hwin = H < pairs ? H : pairs;
+  if (rows < 1 || rows * a.hwin > pairs) return 1;
+  const size_t esz = bf ? 2 : 4;
+  a.kstride = lds_stride(Dk, esz);
+  const size_t smem = lds_bytes(Dk, esz, PW);
+  int rc = 0;
+#define RT_ATTN(CPLv)                                                                              \
+  rc = bf ? (PW == 8 ? launch_one<uint16_t, CPLv, 8>(a, n_tiles, smem, stream)                     \
+                     : launch_one<uint16_t, CPLv, 2>(a, n_tiles, smem, stream))                    \
+          : (PW == 8 ? launch_one<float, CPLv, 8>(a, n_tiles, smem, stream)                        \
+                     : launch_one<float, CPLv, 2>(a, n_tiles, smem, stream))
+  if (C <= 64) RT_ATTN(1);
+  else if (C <= 128) RT_ATTN(2);
+  else if (C <= 256) RT_ATTN(4);
+  else RT_ATTN(8);
+#undef RT_ATTN
+  if (rc == 0 && num_splits > 1) {
+    if (bf) hipLaunchKernelGGL((latent_combine_kernel<uint16_t>), dim3(T, H), dim3(64), 0, stream, (uint16_t*)out, part_o, part_ml, sink, T, H, C, num_splits);
+    else hipLaunchKernelGGL((latent_combine_kernel<float>), dim3(T, H), dim3(64), 0, stream, (float*)out, part_o, part_ml, sink, T, H, C, num_splits);
+  }
+  return rc;
+}

@@ -506,7 +506,9 @@ class Engine:
             self.stats["decode_tokens"] += at if single else 0
             for key in end:
                 self.release(key)
-            return out.float()
+            out = out.float()
+        self._sync()    # the caller reads the logits from another stream (or the host)
+        return out
 
     def _decode_rows(self, spans: Sequence[Tuple[SeqState, int, Sequence[int]]]) -> torch.Tensor:
         """One eager decode-kind forward: span b feeds ONE token at position ``st`` of its sequence."""

@@ -148,7 +148,7 @@ class MupulornModel:
         step (all rows when it is None). ``keep_layers``: a list that receives the residual stream
         after every layer (debugging / tests)."""
         cfg, adt = self.cfg, self.dtype
-        eps, taps = cfg.norm_eps, cfg.canon_taps
+        eps = cfg.norm_eps
         T = ids.shape[0]
         b = self._rows(positions, meta)
         decode = meta.kind == "decode"
@@ -158,14 +158,14 @@ class MupulornModel:
             lw, m = self.layers[ls.source], ls.mixer
             conv, rows = kv.conv[l], kv.layer_rows(l)
             h = L.canon_norm(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.row_seq, positions, b.start_pos, b.slots, adt)
-            L.canon_state_update(x, lw["norm1"], eps, taps, conv, 0, b.cu_q, b.start_pos, b.slots)
+            L.canon_state_update(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.cu_q, b.start_pos, b.slots)
             proj = F.linear(h, lw["w_in"])
             cq = L.latent_prep(proj, m, lw["mix.dq.norm"], lw["mix.dkv.norm"], eps, positions, rows,
                                meta.slot_mapping, adt)
             q = F.linear(cq, lw["mix.uq"]).view(T, m.heads, m.dim + m.rot_dim)
             q_lat = torch.bmm(q[:, :, :m.dim].transpose(0, 1), lw["uk_h"])
             o_lat = L.latent_attention(q_lat, q, m, rows, meta.block_tables, b.cu_q, b.start_pos, lw["mix.sink"],
-                                       tiles=self._tiles(meta, L.rows_per_tile(m.heads, m.kv_rank), b)
+                                       tiles=self._tiles(meta, L.rows_per_tile(m.heads, m.kv_rank, m.rot_dim, adt), b)
                                        if x.is_cuda else None,
                                        num_splits=splits, workspace=self._workspace(T, m, splits), out_dtype=adt)
             o = torch.bmm(o_lat, lw["uv_ht"])
@@ -174,7 +174,7 @@ class MupulornModel:
             if ls.ff:
                 h = L.canon_norm(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.row_seq, positions, b.start_pos,
                                  b.slots, adt)
-                L.canon_state_update(x, lw["norm2"], eps, taps, conv, 1, b.cu_q, b.start_pos, b.slots)
+                L.canon_state_update(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.cu_q, b.start_pos, b.slots)
                 a = L.poly_norm(F.linear(h, lw["mlp.up"]), lw["mlp.act"], eps, adt)
                 L.scalar_norm_add_(x, F.linear(a, lw["mlp.down"]), lw["norm2b"], eps)
             if keep_layers is not None:

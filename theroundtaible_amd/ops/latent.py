@@ -82,13 +82,14 @@ def canon_norm(x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, ou
     return ref.canon_norm(x, g, eps, w, conv[:, sub, :w.shape[1] - 1], row_seq, positions, start_pos, slots, out_dtype)
 
 
-def canon_state_update(x, g, eps, taps, conv, sub, cu_q, start_pos, slots):
-    if taps <= 1:
+def canon_state_update(x, g, eps, w, conv, sub, cu_q, start_pos, slots):
+    """Runs AFTER :func:`canon_norm` of the same sublayer (it overwrites what that one reads)."""
+    if w.shape[1] <= 1:
         return
     if _gpu(x):
-        native().canon_state_update(x, g, float(eps), conv, int(sub), cu_q, start_pos, slots)
+        native().canon_state_update(x, g, float(eps), w, conv, int(sub), cu_q, start_pos, slots)
         return
-    ref.canon_state_update(x, g, eps, conv[:, sub], cu_q, start_pos, slots)
+    ref.canon_state_update(x, g, eps, conv[:, sub, :w.shape[1] - 1], cu_q, start_pos, slots)
 
 
 def latent_prep(proj, spec, wq, wkv, eps, positions, cache_rows, slot_mapping, out_dtype):
@@ -101,10 +102,13 @@ def latent_prep(proj, spec, wq, wkv, eps, positions, cache_rows, slot_mapping, o
                            spec.rot_dims, cache_rows, slot_mapping, out_dtype)
 
 
-def rows_per_tile(heads: int, kv_rank: int) -> int:
-    """Query rows one attention workgroup takes (all heads of each row share the staged key tile)."""
-    pairs = 32 if kv_rank <= 128 else 16 if kv_rank <= 256 else 8
-    return max(1, pairs // min(heads, pairs))
+def rows_per_tile(heads: int, kv_rank: int, rot_dim: int, dtype) -> int:
+    """Query rows one attention workgroup takes (all heads of each row share the staged key tile);
+    the kernel's own rule (it depends on what fits the LDS)."""
+    rows = int(native().latent_rows_per_tile(heads, kv_rank, rot_dim, dtype == torch.bfloat16))
+    if rows <= 0:
+        raise ValueError(f"latent attention: a cached row of {kv_rank + rot_dim} numbers does not fit the kernel's LDS tile")
+    return rows
 
 
 def tile_map(cu_q: torch.Tensor, start_pos: torch.Tensor, rows: int) -> torch.Tensor:
@@ -139,7 +143,7 @@ def latent_attention(q_lat, q, spec, cache_rows, block_tables, cu_q, start_pos, 
         if C > MAX_LATENT:
             raise ValueError(f"latent attention kernels hold at most {MAX_LATENT} latent dims per row, got {C}")
         out = torch.empty(H, T, C, dtype=out_dtype, device=q.device)
-        rows = rows_per_tile(H, C)
+        rows = 1 if num_splits > 1 else rows_per_tile(H, C, q.shape[2] - spec.dim, q.dtype)
         if tiles is None:
             tiles = tile_map(cu_q.cpu(), start_pos.cpu(), rows).to(q.device)
         if num_splits > 1 and workspace is None:
