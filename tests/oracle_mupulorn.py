@@ -62,9 +62,8 @@ def sink_softmax_attention(q, k, v, sink, scale):
     return out
 
 
-def latent_attention(h, P, pre, m, eps):
-    """The mixer: low-rank queries, one shared latent for keys and values, a rotated key part
-    shared by all heads, a per-head sink, an output gate."""
+def latent_qkv(h, P, pre, m, eps):
+    """Per-head queries and keys [H, T, dim + rot_dim] (rotated parts last) and values [H, T, vdim]."""
     T = h.shape[0]
     H, D, R, Dv, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     pos = torch.arange(T)
@@ -76,11 +75,17 @@ def latent_attention(h, P, pre, m, eps):
     q_rot = rotate_pairs(q[:, :, D:], pos, m["rot"]["base"], m["rot"]["dims"])
     kn = (c @ P[pre + "uk"].T).view(T, H, D)
     vv = (c @ P[pre + "uv"].T).view(T, H, Dv)
-    heads = []
-    for hh in range(H):
-        qh = torch.cat([q[:, hh, :D], q_rot[:, hh]], -1)
-        kh = torch.cat([kn[:, hh], k_rot], -1)
-        heads.append(sink_softmax_attention(qh, kh, vv[:, hh], P[pre + "sink"][hh], m["scale"]))
+    qs = torch.stack([torch.cat([q[:, hh, :D], q_rot[:, hh]], -1) for hh in range(H)])
+    ks = torch.stack([torch.cat([kn[:, hh], k_rot], -1) for hh in range(H)])
+    return qs, ks, vv.transpose(0, 1)
+
+
+def latent_attention(h, P, pre, m, eps):
+    """The mixer: low-rank queries, one shared latent for keys and values, a rotated key part
+    shared by all heads, a per-head sink, an output gate."""
+    qs, ks, vs = latent_qkv(h, P, pre, m, eps)
+    heads = [sink_softmax_attention(qs[hh], ks[hh], vs[hh], P[pre + "sink"][hh], m["scale"])
+             for hh in range(m["heads"])]
     o = torch.cat(heads, -1) * torch.sigmoid(h @ P[pre + "g"].T)
     return o @ P[pre + "o"].T
 

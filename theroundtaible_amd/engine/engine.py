@@ -305,7 +305,8 @@ class Engine:
         s = self.kv.seq(key)
         n = lcp(s.tokens, target, len(target) - 1)   # always recompute >= 1 token (need its logits)
         self.kv.truncate(s, n)
-        return s, n
+        # a sequence with a running state can only be kept whole: any other cut restarts it
+        return s, min(n, s.length)
 
     @staticmethod
     def shared_seq_key(key: str) -> str:
@@ -368,7 +369,7 @@ class Engine:
         logits are used. Tensor-parallel engines never speculate (their ranks would have to
         agree on it). Returns the tokens prefilled."""
         key = getattr(prompt, "shared_key", None)
-        if key is None or not self.healthy or self.tp.size > 1:
+        if key is None or not self.healthy or self.tp.size > 1 or getattr(self.model, "stateful", False):
             return 0
         ids, n = self.encode_prompt_split(prompt)
         if n <= 0:
@@ -709,6 +710,9 @@ class Engine:
         Returns (per-turn group key or None, {key: shared seq}, {key: shared prefill tokens},
         reserved shared spans)."""
         keys = [getattr(t.prompt, "shared_key", None) if n > 0 else None for t, (_, n) in zip(turns, enc)]
+        if getattr(self.model, "stateful", False):
+            # shared blocks carry no running state: every member prefills its whole prompt
+            keys = [None] * len(turns)
         shared: Dict[str, SeqState] = {}
         pre: Dict[str, int] = {}
         items = []
