@@ -112,7 +112,78 @@ def parse():
     p.add_argument("--write-calibration", default=None,
                    help="(N > 1) write the node's measured K9 latency / fused saving as a cost-model calibration "
                         "JSON (parallel/costmodel.py default_calibration, $ROUNDTABLE_CALIBRATION)")
+    p.add_argument("--arch-compare", default="",
+                   help="instead of the headline workload: prefill and decode throughput of model pairs "
+                        "'a:b,c:d' (e.g. mupulorn-8b:llama3-8b,mupulorn-1b:llama3.2-1b), each model with "
+                        "--compare-layers layers and random weights, through the same engine entry points; "
+                        "prints one JSON line per model")
+    p.add_argument("--compare-layers", type=int, default=4)
+    p.add_argument("--compare-prompt", type=int, default=4096, help="--arch-compare: prompt tokens per sequence")
+    p.add_argument("--compare-batch", type=int, default=8, help="--arch-compare: sequences decoded together")
+    p.add_argument("--compare-new", type=int, default=128, help="--arch-compare: decoded tokens per sequence")
     return p.parse_args()
+
+
+def _arch_compare(args) -> int:
+    """Prefill and decode throughput of several models at equal layer count, one engine each, the
+    same entry points the serving path uses: ``Engine.prefill`` (varlen, chunked) and
+    ``Engine.continue_decode`` (the captured decode step)."""
+    import torch
+    from theroundtaible_amd.engine.engine import Engine, EngineConfig, Turn
+    from theroundtaible_amd.engine.sampler import SamplingParams
+    from theroundtaible_amd.models.config import get_config
+    device = args.device or "cuda:0"
+    P, B, NEW, L = args.compare_prompt, args.compare_batch, args.compare_new, args.compare_layers
+    for pair in filter(None, args.arch_compare.split(",")):
+        for name in pair.split(":"):
+            base = get_config(name)
+            ov = {"n_layers": L}
+            if base.layers is not None:
+                ov["layers"] = tuple(base.layers[:L])
+            eng = Engine(EngineConfig(model=name, weights=args.weights, device=device, model_overrides=ov,
+                                      dtype="bf16" if device != "cpu" else "fp32",
+                                      use_graphs=not args.no_graphs and device != "cpu",
+                                      max_kv_tokens=B * (P + NEW + 64) + 4096, max_batch=B, state_slots=B))
+            g = torch.Generator().manual_seed(1)
+            prompts = [torch.randint(0, base.vocab, (P,), generator=g).tolist() for _ in range(B)]
+            sp = SamplingParams(temperature=0.0, max_new_tokens=NEW, ignore_eos=True, stop_on_consensus=False)
+            turns = [Turn(f"s{i}", "", sp) for i in range(B)]
+
+            def sync():
+                if device != "cpu":
+                    torch.cuda.synchronize()
+
+            def prefill_all(tag):
+                seqs = [eng.kv.seq(f"{tag}{i}") for i in range(B)]
+                with eng._on_stream():
+                    sync()
+                    t0 = time.perf_counter()
+                    for sq, ids in zip(seqs, prompts):      # one sequence per forward: prompt-bound shapes
+                        eng.prefill([(sq, ids)])
+                    sync()
+                return seqs, time.perf_counter() - t0
+            warm, _ = prefill_all("w")
+            for i in range(B):
+                eng.release(f"w{i}")
+            seqs, t_pre = prefill_all("s")
+            eng.continue_decode(seqs, turns, [1] * B, 8)          # capture + warm-up
+            sync()
+            t0 = time.perf_counter()
+            eng.continue_decode(seqs, turns, [1] * B, NEW)
+            sync()
+            t_dec = time.perf_counter() - t0
+            cfg = eng.cfg
+            print(json.dumps({"metric": "arch compare", "model": name, "layers": L, "params_per_layer_M":
+                              round((cfg.n_params() - 2 * cfg.vocab * cfg.hidden) / L / 1e6, 1),
+                              "prefill_tok_s": round(B * P / t_pre), "prefill_tokens": P,
+                              "decode_tok_s": round(B * NEW / t_dec), "decode_batch": B, "decode_context": P,
+                              "decode_ms_per_step": round(t_dec / NEW * 1e3, 3),
+                              "kv_bytes_per_token_layer": eng.kv_bytes_per_token() // L, "dtype": "bf16",
+                              "data": "synthetic, random-init weights"}), flush=True)
+            del eng, seqs, warm
+            if device != "cpu":
+                torch.cuda.empty_cache()
+    return 0
 
 
 def _self_launch(args) -> int:
@@ -186,6 +257,8 @@ def _failure_line(args, world: int, rec: dict) -> dict:
 
 def main() -> int:
     args = parse()
+    if args.arch_compare:
+        return _arch_compare(args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         return _self_launch(args)
     from theroundtaible_amd.utils import failsafe

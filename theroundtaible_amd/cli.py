@@ -692,6 +692,11 @@ def cmd_serve(args, ui: UI) -> int:
     return 0
 
 
+def cmd_trace(args, ui: UI) -> int:
+    from .trace_run import main as trace_main
+    return trace_main(args.trace_args)
+
+
 # ---- parser -------------------------------------------------------------------------------------
 def _discuss_flags(p):
     g = p.add_mutually_exclusive_group()
@@ -791,6 +796,10 @@ def build_parser() -> argparse.ArgumentParser:
                     help="--tp: seconds one engine operation may take on any rank; a rank past it (or one that "
                          "raises) ends the server with a message naming it (collectives time out a minute later)")
     sv.set_defaults(fn=cmd_serve)
+    tr = sub.add_parser("trace", help="Replay a token trace through the engine and write the logits asked for "
+                                      "(the same program as bin/trace_run)")
+    tr.add_argument("trace_args", nargs=argparse.REMAINDER)
+    tr.set_defaults(fn=cmd_trace)
     b = sub.add_parser("bench", help="Run the roundtable benchmark (wraps bench.py)")
     b.add_argument("bench_args", nargs=argparse.REMAINDER)
     b.set_defaults(fn=cmd_bench)

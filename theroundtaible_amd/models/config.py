@@ -203,8 +203,10 @@ PRESETS.update({
     # a test-sized stack and two whose layers have the shapes of 1B / 8B-class models
     "tiny-mupulorn": mupulorn_config("tiny-mupulorn", 3, 128, 4, 32, 16, 32, 64, 48, 256, 32000, taps=4,
                                      shared_every=2),
-    "mupulorn-1b": mupulorn_config("mupulorn-1b", 16, 2048, 16, 128, 64, 128, 512, 768, 8192, 128256),
-    "mupulorn-8b": mupulorn_config("mupulorn-8b", 32, 4096, 32, 128, 64, 128, 512, 1536, 14336, 128256),
+    # (the two-matrix feed-forward is 1.5x as wide as the gated three-matrix one of the Llama preset
+    # of the same class, so a layer holds about the same weights)
+    "mupulorn-1b": mupulorn_config("mupulorn-1b", 16, 2048, 16, 128, 64, 128, 512, 768, 12288, 128256),
+    "mupulorn-8b": mupulorn_config("mupulorn-8b", 32, 4096, 32, 128, 64, 128, 512, 1536, 21504, 128256),
 })
 
 

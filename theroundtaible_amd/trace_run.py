@@ -43,12 +43,15 @@ def main(argv=None) -> int:
         return 2
     from .engine import Engine, EngineConfig
     from .models.config import get_config
-    if device.startswith("cuda") and get_config(a.model).arch == "mupulorn":
+    from .utils.local_detect import resolve_model
+    # the checkpoint's config.json names the model class, as for every engine built on a directory
+    model, overrides = resolve_model(a.model, a.model)
+    if device.startswith("cuda") and get_config(model, **overrides).arch == "mupulorn":
         from .ops import latent
         latent.ensure_built()          # a fresh checkout compiles this family's kernels here, once
     bs = a.block_size
     live = max(1, a.max_live)
-    engine = Engine(EngineConfig(model=a.model, weights=a.model, dtype=a.dtype, device=device, block_size=bs,
+    engine = Engine(EngineConfig(model=model, model_overrides=overrides, weights=a.model, dtype=a.dtype, device=device, block_size=bs,
                                  num_blocks=(a.max_tokens + bs - 1) // bs, use_graphs=False, state_slots=live,
                                  max_batch=live))
     os.makedirs(a.out, exist_ok=True)

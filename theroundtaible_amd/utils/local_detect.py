@@ -26,7 +26,7 @@ import re
 from dataclasses import dataclass, field
 from typing import Any, Dict, Iterable, List, Optional
 
-from ..models.config import PRESETS
+from ..models.config import ARCHITECTURES, PRESETS
 
 NON_CHAT = re.compile(r"(^|[^a-z])(embed|embedding|tts|whisper|rerank|reranker|clip)([^a-z]|$)", re.I)
 
@@ -139,7 +139,12 @@ def checkpoint_model(path: str) -> Optional[tuple]:
     ``config.json`` alone; None if it is not a recognised Llama / Mistral / Qwen2 / GPT-2 checkpoint."""
     try:
         with open(os.path.join(path, "config.json"), encoding="utf-8") as f:
-            shape = _shape_from_hf(json.load(f))
+            raw = json.load(f)
+        if isinstance(raw, dict) and raw.get("architecture") in ARCHITECTURES:
+            # a per-layer-configured checkpoint: its directory IS the model name (models/config.py
+            # get_config parses the file itself), nothing to override
+            return os.path.abspath(path), {}
+        shape = _shape_from_hf(raw)
     except (OSError, ValueError, KeyError, TypeError):
         return None
     if shape is None:
