@@ -18,6 +18,8 @@
 // follow from the run-time position, so one captured launch serves every length.
 //
 // The rotary part of q is rotated here, on load, by the row's position (fp32 angles).
+#include <cstdlib>
+
 #include "../common.h"
 
 namespace {
@@ -41,6 +43,7 @@ struct AttnArgs {
   float* part_ml;       // [T, H, splits, 2]
   int T, H, C, R, Dq, rot_off, BS, max_blocks, rows, num_splits, kstride, rot_dims;
   int hwin;             // heads one workgroup takes (grid.z walks the windows)
+  int kt;               // keys per staged tile of the plain kernel (64, or fewer when LDS is short)
   float scale, rot_k;
 };
 
@@ -49,8 +52,8 @@ template <typename CT, typename QT, int CPL, int PW>
 __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int Dk = a.C + a.R;
-  CT* Ks = reinterpret_cast<CT*>(smem);                                   // [KT][kstride]
-  float* Qs = reinterpret_cast<float*>(smem + (size_t)KT * a.kstride * sizeof(CT));  // [pairs][Dk]
+  CT* Ks = reinterpret_cast<CT*>(smem);                                   // [kt][kstride]
+  float* Qs = reinterpret_cast<float*>(smem + (size_t)a.kt * a.kstride * sizeof(CT));  // [pairs][Dk]
   float* Ps = Qs + (size_t)kWaves * PW * Dk;                              // [pairs][KT]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seq = a.tiles[blockIdx.x * 2], row0 = a.tiles[blockIdx.x * 2 + 1];
@@ -107,10 +110,11 @@ __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
   }
   const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
   const CT* cache = reinterpret_cast<const CT*>(a.cache);
-  for (int k0 = kb; k0 < ke; k0 += KT) {
+  const int kt = a.kt;
+  for (int k0 = kb; k0 < ke; k0 += kt) {
     __syncthreads();   // the previous tile's readers are done (and Qs is written, first time)
     // stage: wave w copies keys w, w + 4, ...; lanes stride over the row
-    for (int kk = wave; kk < KT; kk += kWaves) {
+    for (int kk = wave; kk < kt; kk += kWaves) {
       const int kp = k0 + kk;
       CT* dst = Ks + (size_t)kk * a.kstride;
       if (kp < ke) {
@@ -125,7 +129,7 @@ __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
     float s[PW];
 #pragma unroll
     for (int i = 0; i < PW; ++i) s[i] = 0.f;
-    const CT* krow = Ks + (size_t)lane * a.kstride;
+    const CT* krow = Ks + (size_t)(lane < kt ? lane : 0) * a.kstride;
     const float* qw = Qs + (size_t)wave * PW * Dk;
     for (int d = 0; d < Dk; ++d) {
       const float kv = DT<CT>::load(krow + d);
@@ -136,7 +140,7 @@ __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
     float* pw = Ps + (size_t)wave * PW * KT;
 #pragma unroll
     for (int i = 0; i < PW; ++i) {
-      const bool vis = kp < ke && kp <= qpos[i];
+      const bool vis = lane < kt && kp < ke && kp <= qpos[i];
       const float sv = vis ? s[i] : -INFINITY;
       const float mn = fmaxf(m[i], rt::wave_max(sv));
       float p = 0.f, alpha = 1.f;
@@ -154,7 +158,7 @@ __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    for (int kk = 0; kk < KT; ++kk) {
+    for (int kk = 0; kk < kt; ++kk) {
       float kvv[CPL];
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
@@ -229,6 +233,218 @@ __global__ void __launch_bounds__(64) latent_combine_kernel(OT* __restrict__ out
   }
 }
 
+// ---- bf16 on the matrix cores ----------------------------------------------------------------
+// Workgroup = 4 waves over 64 (row, head) pairs and a 64-key tile; wave w = (ph, x): ph = w >> 1
+// is its half of the pairs (32 MFMA columns), x = w & 1 its half of the tile's KEYS while scores
+// are formed and its half of the latent COLUMNS while values are accumulated:
+//
+//   stage    lane = key: the tile's rows -> LDS row-major (K), and their latent part transposed
+//            (V^T [C][64 keys]): the value product contracts over keys, the cache row over dims
+//   S^T      [32 keys x 32 pairs] = K . Q^T   Dk/16 x mfma_f32_32x32x16_bf16, Q fragments in
+//            registers; K rows are read with bits 2 and 3 of the row index swapped, which leaves
+//            lane (pair, h) with keys 16j + 8h + 0..7: the B fragment of P^T as it stands
+//   softmax  each lane owns ONE pair: mask by its position, tile maximum over the wave's keys,
+//            exchanged with the other key half through LDS, P -> LDS [pair][key] as bf16
+//   O^T      [C/2 latent cols x 32 pairs] += V^T . P^T   (C/64 blocks x 4 key chunks)
+//
+// Needs C a multiple of 64 (<= 512), R a multiple of 16 (<= 64).
+typedef float f16v __attribute__((ext_vector_type(16)));
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kVRow = KT * 2 + 16;   // bytes per V^T / P row in LDS (64 keys + pad)
+
+RT_DEVICE int swap23(int x) { return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1); }
+
+template <int NB>   // NB = C / 64: 32-column value blocks per wave
+__global__ void __launch_bounds__(kThreads) latent_attn_mfma_kernel(AttnArgs a) {
+  constexpr int NQM = NB * 4 + 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int C = a.C, Dk = a.C + a.R, nq = Dk >> 4;
+  const int krow_b = Dk * 2 + 16;
+  unsigned char* Kt = smem;
+  unsigned char* Vt = Kt + (size_t)KT * krow_b;
+  unsigned char* Pt = Vt + (size_t)C * kVRow;
+  float* mx = reinterpret_cast<float*>(Pt + 64 * kVRow);   // [2][64]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, h = lane >> 5, ph = wave >> 1, x = wave & 1;
+  const int seq = a.tiles[blockIdx.x * 2], row0 = a.tiles[blockIdx.x * 2 + 1];
+  const int nrows = min(a.rows, a.cu_q[seq + 1] - row0);
+  const int pos0 = a.start_pos[seq] + (row0 - a.cu_q[seq]);
+  const int h0 = blockIdx.z * a.hwin;
+  const int HW = min(a.hwin, a.H - h0);
+  const int npairs = nrows * HW;
+  // ---- queries -> LDS (bf16, rotary part rotated), then each lane's B fragments -> registers ----
+  for (int p = wave; p < 64; p += kWaves) {
+    uint16_t* qd = reinterpret_cast<uint16_t*>(Kt + (size_t)p * krow_b);
+    if (p >= npairs) {
+      for (int d = lane; d < Dk; d += 64) qd[d] = 0;
+      continue;
+    }
+    const int r = p / HW, hd = h0 + p - r * HW;
+    const uint16_t* ql = reinterpret_cast<const uint16_t*>(a.q_lat) + ((size_t)hd * a.T + row0 + r) * C;
+    for (int d = lane; d < C; d += 64) qd[d] = ql[d];
+    const uint16_t* qr = reinterpret_cast<const uint16_t*>(a.q) + ((size_t)(row0 + r) * a.H + hd) * a.Dq + a.rot_off;
+    const float posf = (float)(pos0 + r);
+    for (int i = lane; i < a.R / 2; i += 64) {
+      const float u = rt::bf2f(qr[2 * i]), v = rt::bf2f(qr[2 * i + 1]);
+      float cs = 1.f, sn = 0.f;
+      if (2 * i < a.rot_dims) sincosf(posf * exp2f((float)i * a.rot_k), &sn, &cs);
+      qd[C + 2 * i] = rt::f2bf(u * cs - v * sn);
+      qd[C + 2 * i + 1] = rt::f2bf(v * cs + u * sn);
+    }
+  }
+  __syncthreads();
+  rt::short8 qf[NQM];
+#pragma unroll
+  for (int dk = 0; dk < NQM; ++dk)
+    if (dk < nq) qf[dk] = *reinterpret_cast<const rt::short8*>(Kt + (size_t)(ph * 32 + c) * krow_b + 32 * dk + 16 * h);
+  const int mp = ph * 32 + c;                              // this lane's pair
+  const int qpos = mp < npairs ? pos0 + mp / HW : -1;
+  f16v o[NB];
+#pragma unroll
+  for (int db = 0; db < NB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float m = -INFINITY, l = 0.f;   // m in log2 units of the scaled score
+  const float sc2 = a.scale * kLog2e;
+  const int nkeys = pos0 + nrows;
+  int kb = 0, ke = nkeys;
+  if (a.num_splits > 1) {
+    const int ntile = (nkeys + KT - 1) / KT;
+    const int per = (ntile + a.num_splits - 1) / a.num_splits;
+    kb = min(nkeys, (int)blockIdx.y * per * KT);
+    ke = min(nkeys, kb + per * KT);
+  }
+  const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
+  const uint16_t* cache = reinterpret_cast<const uint16_t*>(a.cache);
+  const int nch = Dk >> 3;   // 16-byte chunks per cached row
+  for (int k0 = kb; k0 < ke; k0 += KT) {
+    __syncthreads();   // the previous tile (and the query fragments' source) is consumed
+    {
+      const int kp = k0 + lane;
+      const bool ok = kp < ke;
+      const uint16_t* src = cache + ((size_t)(ok ? bt[kp / a.BS] : 0) * a.BS + (ok ? kp % a.BS : 0)) * Dk;
+      for (int ch = wave; ch < nch; ch += kWaves) {
+        rt::u32x4 v = {0u, 0u, 0u, 0u};
+        if (ok) v = *reinterpret_cast<const rt::u32x4*>(src + ch * 8);
+        *reinterpret_cast<rt::u32x4*>(Kt + (size_t)lane * krow_b + ch * 16) = v;
+        if (ch * 8 < C) {
+          uint16_t* vt = reinterpret_cast<uint16_t*>(Vt + (size_t)(ch * 8) * kVRow) + lane;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            vt[(size_t)(2 * j) * (kVRow / 2)] = (uint16_t)(v[j] & 0xffffu);
+            vt[(size_t)(2 * j + 1) * (kVRow / 2)] = (uint16_t)(v[j] >> 16);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // ---- S^T = K Q^T for this wave's 32 keys x 32 pairs ----
+    f16v sc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+    const unsigned char* kr = Kt + (size_t)(32 * x + swap23(c)) * krow_b + 16 * h;
+#pragma unroll
+    for (int dk = 0; dk < NQM; ++dk)
+      if (dk < nq) {
+        const rt::short8 ka = *reinterpret_cast<const rt::short8*>(kr + 32 * dk);
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rt::bf16x8, ka),
+                                                     __builtin_bit_cast(rt::bf16x8, qf[dk]), sc, 0, 0, 0);
+      }
+    // reg i holds key k0 + 32x + 16 (i >> 3) + 8h + (i & 7) of pair mp
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = k0 + 32 * x + 16 * (i >> 3) + 8 * h + (i & 7);
+      const float v = (key < ke && key <= qpos) ? sc[i] * sc2 : -INFINITY;
+      sc[i] = v;
+      tmax = fmaxf(tmax, v);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    if (h == 0) mx[x * 64 + mp] = tmax;
+    __syncthreads();
+    const float mn = fmaxf(m, fmaxf(mx[mp], mx[64 + mp]));
+    const float msub = (mn == -INFINITY) ? 0.f : mn;
+    const float alpha = (mn == -INFINITY) ? 1.f : exp2f(m - mn);
+    m = mn;
+    float psum = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      rt::u32x4 w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float p0 = exp2f(sc[8 * blk + 2 * j] - msub), p1 = exp2f(sc[8 * blk + 2 * j + 1] - msub);
+        psum += p0 + p1;
+        w[j] = rt::pack2(p0, p1);
+      }
+      *reinterpret_cast<rt::u32x4*>(Pt + (size_t)mp * kVRow + (32 * x + 16 * blk + 8 * h) * 2) = w;
+    }
+    l = l * alpha + psum;
+#pragma unroll
+    for (int db = 0; db < NB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    __syncthreads();
+    // ---- O^T += V^T P^T for this wave's half of the latent columns ----
+    const unsigned char* pr = Pt + (size_t)mp * kVRow + 16 * h;
+#pragma unroll
+    for (int db = 0; db < NB; ++db) {
+      const unsigned char* vr = Vt + (size_t)(x * (C / 2) + 32 * db + c) * kVRow + 16 * h;
+#pragma unroll
+      for (int kc = 0; kc < 4; ++kc) {
+        const rt::short8 va = *reinterpret_cast<const rt::short8*>(vr + 32 * kc);
+        const rt::short8 pb = *reinterpret_cast<const rt::short8*>(pr + 32 * kc);
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(rt::bf16x8, va),
+                                                        __builtin_bit_cast(rt::bf16x8, pb), o[db], 0, 0, 0);
+      }
+    }
+  }
+  // ---- the pair's sum over both key halves, then the sink (or the split partials) ----
+  l += __shfl_xor(l, 32, 64);
+  __syncthreads();
+  if (h == 0) mx[x * 64 + mp] = l;
+  __syncthreads();
+  const float ltot = mx[mp] + mx[64 + mp];
+  if (mp >= npairs) return;
+  const int r = mp / HW, hd = h0 + mp - r * HW, t = row0 + r;
+  const float m_nat = m * kLn2;
+  if (a.num_splits > 1) {
+    float* po = a.part_o + (((size_t)t * a.H + hd) * a.num_splits + blockIdx.y) * C;
+#pragma unroll
+    for (int db = 0; db < NB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) po[x * (C / 2) + 32 * db + 8 * (i >> 2) + 4 * h + (i & 3)] = o[db][i];
+    if (x == 0 && h == 0) {
+      float* ml = a.part_ml + (((size_t)t * a.H + hd) * a.num_splits + blockIdx.y) * 2;
+      ml[0] = m_nat;
+      ml[1] = ltot;
+    }
+  } else {
+    const float sk = a.sink[hd];
+    const float M = fmaxf(m_nat, sk);
+    const float w = __expf(m_nat - M);
+    const float inv = w / (ltot * w + __expf(sk - M));
+    uint16_t* orow = reinterpret_cast<uint16_t*>(a.out) + ((size_t)hd * a.T + t) * C;
+#pragma unroll
+    for (int db = 0; db < NB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        orow[x * (C / 2) + 32 * db + 8 * (i >> 2) + 4 * h + (i & 3)] = rt::f2bf(o[db][i] * inv);
+  }
+}
+
+template <int NB>
+int launch_mfma(const AttnArgs& a, int n_tiles, size_t smem, hipStream_t stream) {
+  auto kern = latent_attn_mfma_kernel<NB>;
+  if (smem > 64 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      return 3;
+  }
+  hipLaunchKernelGGL(kern, dim3(n_tiles, a.num_splits, (a.H + a.hwin - 1) / a.hwin), dim3(kThreads), smem, stream, a);
+  return 0;
+}
+
 template <typename CT, int CPL, int PW>
 int launch_one(const AttnArgs& a, int n_tiles, size_t smem, hipStream_t stream) {
   auto kern = latent_attn_kernel<CT, CT, CPL, PW>;
@@ -250,19 +466,41 @@ static int lds_stride(int Dk, size_t esz) {
   return (int)(words * 4 / esz);
 }
 
-static size_t lds_bytes(int Dk, size_t esz, int PW) {
-  return (size_t)KT * lds_stride(Dk, esz) * esz + (size_t)kWaves * PW * Dk * 4 + (size_t)kWaves * PW * KT * 4;
+static size_t lds_bytes(int Dk, size_t esz, int PW, int kt) {
+  return (size_t)kt * lds_stride(Dk, esz) * esz + (size_t)kWaves * PW * Dk * 4 + (size_t)kWaves * PW * KT * 4;
 }
 
-// (row, head) pairs per wave: 8 when the staged tile, the queries and the weights fit the 160 KB
-// of LDS, else 2; 0: the row is too wide for this kernel
-static int pairs_per_wave(int Dk, bool bf) {
+// (row, head) pairs per wave and keys per staged tile of the plain kernel: 8 pairs and 64 keys
+// when the tile, the queries and the weights fit the 160 KB of LDS, else fewer keys, then fewer
+// pairs; 0: the row is too wide for this kernel
+static int pairs_per_wave(int Dk, bool bf, int* kt_out = nullptr) {
   const size_t esz = bf ? 2 : 4, cap = 160 * 1024;
-  return lds_bytes(Dk, esz, 8) <= cap ? 8 : lds_bytes(Dk, esz, 2) <= cap ? 2 : 0;
+  const int cand[5][2] = {{8, 64}, {8, 32}, {2, 64}, {2, 32}, {2, 16}};
+  for (auto& pk : cand)
+    if (lds_bytes(Dk, esz, pk[0], pk[1]) <= cap) {
+      if (kt_out) *kt_out = pk[1];
+      return pk[0];
+    }
+  return 0;
+}
+
+static size_t mfma_lds_bytes(int C, int R) {
+  return (size_t)KT * ((C + R) * 2 + 16) + (size_t)C * kVRow + 64 * kVRow + 2 * 64 * sizeof(float);
+}
+
+// the matrix-core kernel takes bf16 rows whose latent is a multiple of 64 (1, 2, 3, 4, 6 or 8
+// times) and whose rotary part is a multiple of 16 up to 64; ROUNDTABLE_LATENT_FMA=1 pins the
+// plain kernel (A/B)
+static bool use_mfma(int C, int R, bool bf) {
+  static const bool off = [] { const char* e = getenv("ROUNDTABLE_LATENT_FMA"); return e && e[0] == '1'; }();
+  const int nb = C / 64;
+  return bf && !off && C % 64 == 0 && (nb == 1 || nb == 2 || nb == 3 || nb == 4 || nb == 6 || nb == 8) &&
+         R % 16 == 0 && R <= 64 && mfma_lds_bytes(C, R) <= 160 * 1024;
 }
 
 // query rows per workgroup: all heads of a row (up to the workgroup's pairs) share the key tile
 int latent_rows_per_tile(int H, int C, int R, bool bf) {
+  if (use_mfma(C, R, bf)) return H >= 64 ? 1 : 64 / H;
   const int pairs = kWaves * pairs_per_wave(C + R, bf);
   if (pairs == 0) return 0;
   return H >= pairs ? 1 : pairs / H;
@@ -277,7 +515,9 @@ int launch_latent_attention(void* out, const void* q_lat, const void* q, const v
   if (n_tiles <= 0 || T <= 0) return 0;
   if (C > 512) return 2;
   const int Dk = C + R;
-  const int PW = pairs_per_wave(Dk, bf);
+  const bool mfma = use_mfma(C, R, bf);
+  int kt = KT;
+  const int PW = mfma ? 16 : pairs_per_wave(Dk, bf, &kt);
   if (PW == 0) return 3;
   const int pairs = kWaves * PW;
   AttnArgs a;
@@ -287,11 +527,23 @@ int launch_latent_attention(void* out, const void* q_lat, const void* q, const v
   a.rows = rows; a.num_splits = num_splits; a.rot_dims = rot_dims; a.scale = scale;
   a.rot_k = rot_dims > 0 ? (float)(-2.0 * log2((double)rot_base) / rot_dims) : 0.f;
   a.hwin = H < pairs ? H : pairs;
+  a.kt = kt;
   if (rows < 1 || rows * a.hwin > pairs) return 1;
   const size_t esz = bf ? 2 : 4;
   a.kstride = lds_stride(Dk, esz);
-  const size_t smem = lds_bytes(Dk, esz, PW);
+  const size_t smem = mfma ? 0 : lds_bytes(Dk, esz, PW, kt);
   int rc = 0;
+  if (mfma) {
+    const size_t sm = mfma_lds_bytes(C, R);
+    switch (C / 64) {
+      case 1: rc = launch_mfma<1>(a, n_tiles, sm, stream); break;
+      case 2: rc = launch_mfma<2>(a, n_tiles, sm, stream); break;
+      case 3: rc = launch_mfma<3>(a, n_tiles, sm, stream); break;
+      case 4: rc = launch_mfma<4>(a, n_tiles, sm, stream); break;
+      case 6: rc = launch_mfma<6>(a, n_tiles, sm, stream); break;
+      default: rc = launch_mfma<8>(a, n_tiles, sm, stream); break;
+    }
+  } else {
 #define RT_ATTN(CPLv)                                                                              \
   rc = bf ? (PW == 8 ? launch_one<uint16_t, CPLv, 8>(a, n_tiles, smem, stream)                     \
                      : launch_one<uint16_t, CPLv, 2>(a, n_tiles, smem, stream))                    \
@@ -302,6 +554,7 @@ int launch_latent_attention(void* out, const void* q_lat, const void* q, const v
   else if (C <= 256) RT_ATTN(4);
   else RT_ATTN(8);
 #undef RT_ATTN
+  }
   if (rc == 0 && num_splits > 1) {
     if (bf) hipLaunchKernelGGL((latent_combine_kernel<uint16_t>), dim3(T, H), dim3(64), 0, stream, (uint16_t*)out, part_o, part_ml, sink, T, H, C, num_splits);
     else hipLaunchKernelGGL((latent_combine_kernel<float>), dim3(T, H), dim3(64), 0, stream, (float*)out, part_o, part_ml, sink, T, H, C, num_splits);

@@ -108,7 +108,10 @@ def _attention_case(dtype, m, lens, starts, BS, seed, splits=1):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(8, 64, 16, 128), (3, 24, 10, 72), (5, 32, 0, 200), (40, 16, 8, 64), (2, 64, 32, 320)])
+@pytest.mark.parametrize("shape", [(8, 64, 16, 128), (3, 24, 10, 72), (5, 32, 0, 200), (40, 16, 8, 64), (2, 64, 32, 320),
+                                   # bf16 shapes of the matrix-core kernel: latent 64 .. 512, rotary 0 .. 64, more
+                                   # heads than one workgroup's 64 pairs
+                                   (16, 128, 64, 512), (70, 32, 16, 64), (3, 32, 32, 192), (4, 16, 0, 256), (6, 32, 48, 384)])
 def test_latent_attention_varlen(dtype, shape):
     H, D, R, C = shape
     m = _spec(H, D, R, 16, C, 32)
@@ -117,8 +120,10 @@ def test_latent_attention_varlen(dtype, shape):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("splits", [2, 7, 32])
-def test_latent_attention_split_keys(dtype, splits):
-    m = _spec(6, 32, 16, 16, 96, 32)
+@pytest.mark.parametrize("shape", [(6, 32, 16, 96), (6, 32, 16, 128), (66, 16, 32, 512)])
+def test_latent_attention_split_keys(dtype, splits, shape):
+    H, D, R, C = shape
+    m = _spec(H, D, R, 16, C, 32)
     _attention_case(dtype, m, [1, 1, 1, 1], [0, 63, 64, 700], 32, seed=splits, splits=splits)
 
 
