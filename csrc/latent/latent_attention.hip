@@ -207,26 +207,35 @@ __global__ void __launch_bounds__(kThreads) latent_attn_kernel(AttnArgs a) {
   }
 }
 
-// one wave per (row, head): merge the split partials and the sink
+// one workgroup per (row, head): merge the split partials and the sink. The splits' weights are
+// formed once (LDS), then every lane sums its columns over the splits with coalesced loads.
 template <typename OT>
-__global__ void __launch_bounds__(64) latent_combine_kernel(OT* __restrict__ out, const float* __restrict__ part_o,
-                                                            const float* __restrict__ part_ml,
-                                                            const float* __restrict__ sink, int T, int H, int C,
-                                                            int splits) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ void __launch_bounds__(256) latent_combine_kernel(OT* __restrict__ out, const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml,
+                                                             const float* __restrict__ sink, int T, int H, int C,
+                                                             int splits) {
+  __shared__ float wgt[64];
+  __shared__ float inv_s;
+  const int t = blockIdx.x, h = blockIdx.y;
   const float* ml = part_ml + ((size_t)t * H + h) * splits * 2;
-  const float sk = sink[h];
-  float M = sk;
-  for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[2 * s]);
-  float den = __expf(sk - M);
-  for (int s = 0; s < splits; ++s) den += ml[2 * s + 1] * __expf(ml[2 * s] - M);   // l = 0 where m = -inf
-  const float inv = 1.f / den;
+  if (threadIdx.x < 64) {
+    const int s = threadIdx.x;
+    const float sk = sink[h];
+    const float ms = s < splits ? ml[2 * s] : -INFINITY;
+    const float M = fmaxf(rt::wave_max(ms), sk);
+    const float w = s < splits ? __expf(ms - M) : 0.f;          // m = -inf (an empty split) -> 0
+    const float den = rt::wave_sum(s < splits ? ml[2 * s + 1] * w : 0.f) + __expf(sk - M);
+    wgt[s] = w;
+    if (s == 0) inv_s = 1.f / den;
+  }
+  __syncthreads();
+  const float inv = inv_s;
   const float* po = part_o + ((size_t)t * H + h) * splits * C;
   OT* orow = out + ((size_t)h * T + t) * C;
-  for (int c = lane; c < C; c += 64) {
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float acc = 0.f;
     for (int s = 0; s < splits; ++s) {
-      const float w = __expf(ml[2 * s] - M);
+      const float w = wgt[s];
       if (w > 0.f) acc += po[(size_t)s * C + c] * w;
     }
     DT<OT>::store(orow + c, acc * inv);
@@ -556,8 +565,8 @@ int launch_latent_attention(void* out, const void* q_lat, const void* q, const v
 #undef RT_ATTN
   }
   if (rc == 0 && num_splits > 1) {
-    if (bf) hipLaunchKernelGGL((latent_combine_kernel<uint16_t>), dim3(T, H), dim3(64), 0, stream, (uint16_t*)out, part_o, part_ml, sink, T, H, C, num_splits);
-    else hipLaunchKernelGGL((latent_combine_kernel<float>), dim3(T, H), dim3(64), 0, stream, (float*)out, part_o, part_ml, sink, T, H, C, num_splits);
+    if (bf) hipLaunchKernelGGL((latent_combine_kernel<uint16_t>), dim3(T, H), dim3(C >= 256 ? 256 : 64), 0, stream, (uint16_t*)out, part_o, part_ml, sink, T, H, C, num_splits);
+    else hipLaunchKernelGGL((latent_combine_kernel<float>), dim3(T, H), dim3(C >= 256 ? 256 : 64), 0, stream, (float*)out, part_o, part_ml, sink, T, H, C, num_splits);
   }
   return rc;
 }

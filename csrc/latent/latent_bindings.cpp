@@ -143,7 +143,7 @@ void latent_attention(torch::Tensor out, torch::Tensor q_lat, torch::Tensor q, i
   chk_i32(tiles, "tiles");
   TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) == start_pos.numel(), "latent_attention: block_tables [S, n]");
   TORCH_CHECK(tiles.dim() == 2 && tiles.size(1) == 2, "latent_attention: tiles [n, 2]");
-  TORCH_CHECK(num_splits >= 1, "latent_attention: num_splits");
+  TORCH_CHECK(num_splits >= 1 && num_splits <= 64, "latent_attention: num_splits must be 1..64");
   float *po = nullptr, *pml = nullptr;
   if (num_splits > 1) {
     TORCH_CHECK(rows == 1, "latent_attention: split keys need one row per tile");
