@@ -333,3 +333,28 @@ def test_rollback_restarts_a_stateful_sequence(tmp_path):
     o = e.run_turns([Turn("A", "Een eerste korte vraag.", sp)])[0]
     assert o.error is None and o.metrics["reused_tokens"] == 0
     assert o.ids == _greedy_oracle(P, cfg, e.encode_prompt("Een eerste korte vraag."), 6)
+
+
+@GPU
+def test_decode_steps_on_the_skinny_gemm(tmp_path):
+    """Sizes the framework's skinny decode GEMM takes (K a multiple of 32, N of 16): decode steps
+    run all five linears of a layer on it, and the logits still match the oracle and the same
+    steps on the library GEMM."""
+    from theroundtaible_amd import ops
+    if not ops.native_available():
+        pytest.skip("main extension not built")
+    lay = [{"type": "latent_attention", "mixer": mixer(2, 16, 16, 16, 64, 32), "mlp": {"kind": "dense", "ff": 96}}] * 2
+    cfg = make_config(width=64, vocab=80, layers=lay)
+    P = make_checkpoint(tmp_path / "m", cfg, seed=11)
+    t = toks(60, cfg["vocab"], 11)
+    want = oracle_logits(P, cfg, t)
+    outs = []
+    for skinny in (True, False):
+        e = engine_for(tmp_path / "m", ("cuda:0", "bf16"))
+        e.model.use_skinny = skinny
+        got = torch.cat([e.step([("a", t[:20], list(range(20)))])] + [e.step([("a", [x], [0])]) for x in t[20:]])
+        close(got, want, ("cuda:0", "bf16"), f"skinny={skinny}")
+        outs.append(got)
+        if skinny:
+            assert all(len(d) == 5 for d in e.model._dec.values())
+    assert float((outs[0] - outs[1]).abs().max()) < 0.2

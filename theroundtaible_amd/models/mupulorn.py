@@ -45,7 +45,12 @@ class _Rows:
     slots: torch.Tensor
 
 
+def x_is_cuda(t: torch.Tensor) -> bool:
+    return t.is_cuda
+
+
 class MupulornModel:
+    use_skinny = True          # decode steps run their linears on the skinny decode GEMM (A/B knob)
     accepts_hidden = False
     stateful = True            # keeps a per-sequence running state beside the paged cache
 
@@ -81,6 +86,8 @@ class MupulornModel:
                     lw[n] = lw[n].to(f32).contiguous()
             self.layers[i] = lw
         self.final_norm = weights["final.norm"].to(f32)
+        self._dec: Optional[Dict[int, Dict[str, torch.Tensor]]] = None
+        self._split_ws: Optional[torch.Tensor] = None
         self._static: Dict[int, tuple] = {}
         self._ws: Dict[tuple, L.LatentWorkspace] = {}
 
@@ -99,6 +106,40 @@ class MupulornModel:
 
     def cache_bytes_per_block(self, block_size: int, dtype_bytes: int) -> int:
         return sum(self.cache_row_dims()) * block_size * dtype_bytes
+
+    # ---- decode GEMMs -----------------------------------------------------------------------------
+    _DEC_LINEARS = ("w_in", "mix.uq", "mix.o", "mlp.up", "mlp.down")
+
+    def decode_weights(self, drop_originals: bool = False) -> Dict[int, Dict[str, torch.Tensor]]:
+        """Fragment-shuffled copies of the five linears of a layer for the framework's skinny decode
+        GEMM (csrc/gemm_skinny.hip: every wave load reads 1 KiB of contiguous weights), built once.
+        Only on a GPU, in bf16, when the main extension is built and the shapes fit its tiles
+        (K a multiple of 32, N of 16); a linear that does not fit keeps its row-major GEMM. The
+        row-major tensors always stay (prompts use them): ``drop_originals`` is not honoured."""
+        if self._dec is None:
+            from .. import ops
+            self._dec = {}
+            ok = self.device.type == "cuda" and self.dtype == torch.bfloat16 and ops.native_available()
+            for i, lw in self.layers.items():
+                d = {}
+                for n in self._DEC_LINEARS if ok else ():
+                    W = lw.get(n)
+                    if W is not None and W.shape[1] % 32 == 0 and W.shape[0] % 16 == 0:
+                        d[n] = ops.shuffle_weight(W)
+                self._dec[i] = d
+            if ok:
+                self._split_ws = ops.split_workspace(self.device)
+        return self._dec
+
+    def _linear(self, x: torch.Tensor, layer: int, name: str, skinny: bool) -> torch.Tensor:
+        """x @ W^T: the skinny decode GEMM for a decode step of up to 32 rows, else the library GEMM."""
+        if skinny:
+            Ws = self._dec[layer].get(name)
+            if Ws is not None:
+                from .. import ops
+                return ops.skinny_gemm(x, Ws, ops.PRO_PLAIN, ops.EPI_STORE, split_ws=self._split_ws,
+                                       split_mode=ops.SPLIT_K | ops.SPLIT_BALANCE)
+        return F.linear(x, self.layers[layer][name])
 
     # ---- forward ----------------------------------------------------------------------------------
     def _rows(self, positions: torch.Tensor, meta: AttnMeta) -> _Rows:
@@ -153,16 +194,17 @@ class MupulornModel:
         b = self._rows(positions, meta)
         decode = meta.kind == "decode"
         splits = self.decode_splits(T) if decode else 1
+        skinny = decode and T <= 32 and x_is_cuda(ids) and self.use_skinny and bool(self.decode_weights())
         x = F.embedding(ids, self.w["embed"]).float()
         for l, ls in enumerate(cfg.layers):
             lw, m = self.layers[ls.source], ls.mixer
             conv, rows = kv.conv[l], kv.layer_rows(l)
             h = L.canon_norm(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.row_seq, positions, b.start_pos, b.slots, adt)
             L.canon_state_update(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.cu_q, b.start_pos, b.slots)
-            proj = F.linear(h, lw["w_in"])
+            proj = self._linear(h, ls.source, "w_in", skinny)
             cq = L.latent_prep(proj, m, lw["mix.dq.norm"], lw["mix.dkv.norm"], eps, positions, rows,
                                meta.slot_mapping, adt)
-            q = F.linear(cq, lw["mix.uq"]).view(T, m.heads, m.dim + m.rot_dim)
+            q = self._linear(cq, ls.source, "mix.uq", skinny).view(T, m.heads, m.dim + m.rot_dim)
             q_lat = torch.bmm(q[:, :, :m.dim].transpose(0, 1), lw["uk_h"])
             o_lat = L.latent_attention(q_lat, q, m, rows, meta.block_tables, b.cu_q, b.start_pos, lw["mix.sink"],
                                        tiles=self._tiles(meta, L.rows_per_tile(m.heads, m.kv_rank, m.rot_dim, adt), b)
@@ -170,13 +212,13 @@ class MupulornModel:
                                        num_splits=splits, workspace=self._workspace(T, m, splits), out_dtype=adt)
             o = torch.bmm(o_lat, lw["uv_ht"])
             og = L.gate_mul(o, proj, m.q_rank + m.cache_row, adt)
-            L.scalar_norm_add_(x, F.linear(og, lw["mix.o"]), lw["norm1b"], eps)
+            L.scalar_norm_add_(x, self._linear(og, ls.source, "mix.o", skinny), lw["norm1b"], eps)
             if ls.ff:
                 h = L.canon_norm(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.row_seq, positions, b.start_pos,
                                  b.slots, adt)
                 L.canon_state_update(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.cu_q, b.start_pos, b.slots)
-                a = L.poly_norm(F.linear(h, lw["mlp.up"]), lw["mlp.act"], eps, adt)
-                L.scalar_norm_add_(x, F.linear(a, lw["mlp.down"]), lw["norm2b"], eps)
+                a = L.poly_norm(self._linear(h, ls.source, "mlp.up", skinny), lw["mlp.act"], eps, adt)
+                L.scalar_norm_add_(x, self._linear(a, ls.source, "mlp.down", skinny), lw["norm2b"], eps)
             if keep_layers is not None:
                 keep_layers.append(x.clone())
         if not decode and meta.last_rows is not None:
