@@ -174,7 +174,8 @@ def _arch_compare(args) -> int:
             t_dec = time.perf_counter() - t0
             cfg = eng.cfg
             print(json.dumps({"metric": "arch compare", "model": name, "layers": L, "params_per_layer_M":
-                              round((cfg.n_params() - 2 * cfg.vocab * cfg.hidden) / L / 1e6, 1),
+                              round((cfg.n_params() - (1 if cfg.tie_embeddings and cfg.layers is None else 2)
+                                     * cfg.vocab * cfg.hidden) / L / 1e6, 1),
                               "prefill_tok_s": round(B * P / t_pre), "prefill_tokens": P,
                               "decode_tok_s": round(B * NEW / t_dec), "decode_batch": B, "decode_context": P,
                               "decode_ms_per_step": round(t_dec / NEW * 1e3, 3),

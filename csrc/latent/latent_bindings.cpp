@@ -10,9 +10,9 @@ void launch_scalar_rms_norm(void* out, const void* x, const float* g, int rows, 
                             bool out_bf, hipStream_t stream);
 void launch_scalar_norm_add(float* res, const void* y, const float* g, int rows, int W, float eps, bool y_bf,
                             hipStream_t stream);
-void launch_canon_norm(void* out, const float* x, const float* g, float eps, const float* w, const float* conv, int sub,
+void launch_canon_norm(void* out, const float* x, const float* g, float eps, const float* w, float* conv, int sub,
                        const int* row_seq, const int64_t* positions, const int* start_pos, const int* slots, int T,
-                       int W, int taps, int keep, bool out_bf, hipStream_t stream);
+                       int W, int taps, int keep, bool out_bf, bool shift_state, hipStream_t stream);
 void launch_canon_state(const float* x, const float* g, float eps, float* conv, int sub, const int* cu_q,
                         const int* start_pos, const int* slots, int S, int W, int taps, int keep, hipStream_t stream);
 void launch_latent_prep(void* cq, const void* proj, int proj_stride, int T, int q_rank, int kv_rank, int rot_dim,
@@ -83,16 +83,18 @@ void chk_conv(const torch::Tensor& conv, const torch::Tensor& w, int64_t W, int6
 
 void canon_norm(torch::Tensor out, torch::Tensor x, torch::Tensor g, double eps, torch::Tensor w, torch::Tensor conv,
                 int64_t sub, torch::Tensor row_seq, torch::Tensor positions, torch::Tensor start_pos,
-                torch::Tensor slots) {
+                torch::Tensor slots, bool shift_state) {
   chk_act(out, "out"); chk_f32(x, "x"); chk_f32(g, "g");
   TORCH_CHECK(x.dim() == 2 && out.sizes() == x.sizes() && g.numel() == 1, "canon_norm: shapes");
   const int64_t T = x.size(0), W = x.size(1);
   chk_conv(conv, w, W, sub);
   chk_i32(row_seq, "row_seq", T); chk_i64(positions, "positions", T);
   chk_i32(start_pos, "start_pos"); chk_i32(slots, "slots", start_pos.numel());
+  // shifting the state in the same launch is only sound with ONE row per sequence
+  TORCH_CHECK(!shift_state || start_pos.numel() == T, "canon_norm: shift_state needs one row per sequence");
   launch_canon_norm(out.data_ptr(), x.data_ptr<float>(), g.data_ptr<float>(), (float)eps, w.data_ptr<float>(),
                     conv.data_ptr<float>(), (int)sub, row_seq.data_ptr<int>(), positions.data_ptr<int64_t>(),
-                    start_pos.data_ptr<int>(), slots.data_ptr<int>(), T, W, w.size(1), conv.size(2), is_bf(out), cur());
+                    start_pos.data_ptr<int>(), slots.data_ptr<int>(), T, W, w.size(1), conv.size(2), is_bf(out), shift_state, cur());
 }
 
 void canon_state_update(torch::Tensor x, torch::Tensor g, double eps, torch::Tensor w, torch::Tensor conv, int64_t sub,

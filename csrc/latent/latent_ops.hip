@@ -56,15 +56,15 @@ __global__ void __launch_bounds__(1024) scalar_norm_add_kernel(float* __restrict
 template <typename OT>
 __global__ void __launch_bounds__(1024) canon_norm_kernel(
     OT* __restrict__ out, const float* __restrict__ x, const float* __restrict__ g, float eps,
-    const float* __restrict__ w, const float* __restrict__ conv, int sub, const int* __restrict__ row_seq,
+    const float* __restrict__ w, float* __restrict__ conv, int sub, const int* __restrict__ row_seq,
     const int64_t* __restrict__ positions, const int* __restrict__ start_pos, const int* __restrict__ slots, int W,
-    int taps, int keep) {
+    int taps, int keep, int shift_state) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const int s = row_seq[t];
   const int64_t pos = positions[t];
   const int local = (int)(pos - start_pos[s]);
-  const float* st = conv + ((size_t)slots[s] * 2 + sub) * keep * W;
+  float* st = conv + ((size_t)slots[s] * 2 + sub) * keep * W;
   // tap k reads the input k rows back: from this batch (local >= k), from the state, or zero
   float inv[kMaxTaps];
   const float* src[kMaxTaps];
@@ -95,6 +95,12 @@ __global__ void __launch_bounds__(1024) canon_norm_kernel(
     for (int k = 0; k < taps; ++k)
       if (src[k] != nullptr) acc += w[(size_t)c * taps + (taps - 1 - k)] * (src[k][c] * inv[k]);
     DT<OT>::store(o + c, acc);
+    if (shift_state) {
+      // one row per sequence (a decode step): this workgroup is the only reader of the sequence's
+      // state, and a lane has read its column's old rows above, so it shifts the column here
+      for (int i = 0; i + 2 < taps; ++i) st[(size_t)i * W + c] = (pos - (taps - 2 - i) >= 0) ? st[(size_t)(i + 1) * W + c] : 0.f;
+      if (taps > 1) st[(size_t)(taps - 2) * W + c] = h0;
+    }
   }
 }
 
@@ -253,12 +259,12 @@ void launch_scalar_norm_add(float* res, const void* y, const float* g, int rows,
   else RT_LAUNCH_W((scalar_norm_add_kernel<float>), rows, W, res, (const float*)y, g, W, eps);
 }
 
-void launch_canon_norm(void* out, const float* x, const float* g, float eps, const float* w, const float* conv, int sub,
+void launch_canon_norm(void* out, const float* x, const float* g, float eps, const float* w, float* conv, int sub,
                        const int* row_seq, const int64_t* positions, const int* start_pos, const int* slots, int T,
-                       int W, int taps, int keep, bool out_bf, hipStream_t stream) {
+                       int W, int taps, int keep, bool out_bf, bool shift_state, hipStream_t stream) {
   if (T <= 0) return;
-  if (out_bf) RT_LAUNCH_W((canon_norm_kernel<uint16_t>), T, W, (uint16_t*)out, x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, W, taps, keep);
-  else RT_LAUNCH_W((canon_norm_kernel<float>), T, W, (float*)out, x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, W, taps, keep);
+  if (out_bf) RT_LAUNCH_W((canon_norm_kernel<uint16_t>), T, W, (uint16_t*)out, x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, W, taps, keep, shift_state ? 1 : 0);
+  else RT_LAUNCH_W((canon_norm_kernel<float>), T, W, (float*)out, x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, W, taps, keep, shift_state ? 1 : 0);
 }
 
 void launch_canon_state(const float* x, const float* g, float eps, float* conv, int sub, const int* cu_q,

@@ -142,3 +142,23 @@ def test_gate_poly_softcap(dtype):
     lg = (torch.randn(T, 1000, generator=g) * 40).to(dtype)
     torch.testing.assert_close(L.logit_softcap(lg.to(DEV), 0.5, 30.0).cpu(), ref.logit_softcap(lg, 0.5, 30.0),
                                rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_canon_norm_shifts_state_in_decode_steps(taps):
+    """One row per sequence: the fused launch gives the output AND the state of the two-launch form."""
+    g = torch.Generator().manual_seed(taps)
+    W, starts = 200, [0, 5, 1, 2, 300]
+    cu, sp, row_seq, pos = _rows_meta([1] * 5, starts)
+    x = torch.randn(5, W, generator=g)
+    w = torch.randn(W, taps, generator=g) * 0.3
+    conv = torch.randn(6, 2, max(taps - 1, 1), W, generator=g)
+    slots = torch.tensor([4, 0, 2, 5, 1], dtype=torch.int32)
+    gain = torch.tensor(0.8)
+    cc = conv.clone()
+    want = L.canon_norm(x, gain, 1e-5, w, cc, 1, row_seq, pos, sp, slots, torch.float32, shift_state=True)
+    cd = conv.clone().to(DEV)
+    got = L.canon_norm(x.to(DEV), gain.to(DEV), 1e-5, w.to(DEV), cd, 1, row_seq.to(DEV), pos.to(DEV), sp.to(DEV),
+                       slots.to(DEV), torch.float32, shift_state=True)
+    torch.testing.assert_close(got.cpu(), want, rtol=2e-4, atol=2e-5)
+    torch.testing.assert_close(cd.cpu(), cc, rtol=1e-5, atol=1e-6)

@@ -199,8 +199,11 @@ class MupulornModel:
         for l, ls in enumerate(cfg.layers):
             lw, m = self.layers[ls.source], ls.mixer
             conv, rows = kv.conv[l], kv.layer_rows(l)
-            h = L.canon_norm(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.row_seq, positions, b.start_pos, b.slots, adt)
-            L.canon_state_update(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.cu_q, b.start_pos, b.slots)
+            # (a decode step shifts the convolution state inside the same launch)
+            h = L.canon_norm(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.row_seq, positions, b.start_pos, b.slots, adt,
+                             shift_state=decode)
+            if not decode:
+                L.canon_state_update(x, lw["norm1"], eps, lw["canon1"], conv, 0, b.cu_q, b.start_pos, b.slots)
             proj = self._linear(h, ls.source, "w_in", skinny)
             cq = L.latent_prep(proj, m, lw["mix.dq.norm"], lw["mix.dkv.norm"], eps, positions, rows,
                                meta.slot_mapping, adt)
@@ -215,8 +218,9 @@ class MupulornModel:
             L.scalar_norm_add_(x, self._linear(og, ls.source, "mix.o", skinny), lw["norm1b"], eps)
             if ls.ff:
                 h = L.canon_norm(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.row_seq, positions, b.start_pos,
-                                 b.slots, adt)
-                L.canon_state_update(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.cu_q, b.start_pos, b.slots)
+                                 b.slots, adt, shift_state=decode)
+                if not decode:
+                    L.canon_state_update(x, lw["norm2"], eps, lw["canon2"], conv, 1, b.cu_q, b.start_pos, b.slots)
                 a = L.poly_norm(self._linear(h, ls.source, "mlp.up", skinny), lw["mlp.act"], eps, adt)
                 L.scalar_norm_add_(x, self._linear(a, ls.source, "mlp.down", skinny), lw["norm2b"], eps)
             if keep_layers is not None:

@@ -73,13 +73,20 @@ def scalar_norm_add_(res, y, g, eps):
     return ref.scalar_norm_add_(res, y, g, eps)
 
 
-def canon_norm(x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, out_dtype):
-    """``conv`` [n_slots, 2, taps - 1, W] fp32, ``sub`` 0 (mixer) / 1 (feed-forward)."""
+def canon_norm(x, g, eps, w, conv, sub, row_seq, positions, start_pos, slots, out_dtype, shift_state=False):
+    """``conv`` [n_slots, 2, taps - 1, W] fp32, ``sub`` 0 (mixer) / 1 (feed-forward).
+    ``shift_state`` (only with ONE row per sequence, a decode step): the same launch also shifts
+    every sequence's state by its row, so no :func:`canon_state_update` follows."""
     if _gpu(x):
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-        native().canon_norm(out, x, g, float(eps), w, conv, int(sub), row_seq, positions, start_pos, slots)
+        native().canon_norm(out, x, g, float(eps), w, conv, int(sub), row_seq, positions, start_pos, slots,
+                            bool(shift_state))
         return out
-    return ref.canon_norm(x, g, eps, w, conv[:, sub, :w.shape[1] - 1], row_seq, positions, start_pos, slots, out_dtype)
+    out = ref.canon_norm(x, g, eps, w, conv[:, sub, :w.shape[1] - 1], row_seq, positions, start_pos, slots, out_dtype)
+    if shift_state and w.shape[1] > 1:
+        cu = torch.arange(x.shape[0] + 1, dtype=torch.int32)
+        ref.canon_state_update(x, g, eps, conv[:, sub, :w.shape[1] - 1], cu, start_pos, slots)
+    return out
 
 
 def canon_state_update(x, g, eps, w, conv, sub, cu_q, start_pos, slots):
