@@ -108,7 +108,7 @@ def _attention_case(dtype, m, lens, starts, BS, seed, splits=1):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(8, 64, 16, 128), (3, 24, 10, 72), (5, 32, 0, 200), (40, 16, 8, 64), (2, 64, 32, 320),
+@pytest.mark.parametrize("shape", [(4, 48, 32, 128), (3, 24, 10, 72), (5, 32, 0, 200), (40, 16, 8, 64), (2, 64, 32, 320),
                                    # bf16 shapes of the matrix-core kernel: latent 64 .. 512, rotary 0 .. 64, more
                                    # heads than one workgroup's 64 pairs
                                    (16, 128, 64, 512), (70, 32, 16, 64), (3, 32, 32, 192), (4, 16, 0, 256), (6, 32, 48, 384)])

@@ -358,3 +358,24 @@ def test_decode_steps_on_the_skinny_gemm(tmp_path):
         if skinny:
             assert all(len(d) == 5 for d in e.model._dec.values())
     assert float((outs[0] - outs[1]).abs().max()) < 0.2
+
+
+def test_serving_entry_points_match_run_turns():
+    """The continuous-batching entry points (prefill + first token, then decode in chunks while the
+    state follows) give the tokens of a single run_turns call; random-init preset weights."""
+    def eng():
+        return Engine(EngineConfig(model="tiny-mupulorn", weights="random:3", dtype="fp32", device="cpu",
+                                   num_blocks=64, use_graphs=False, state_slots=4))
+    sp = SamplingParams(temperature=0.0, max_new_tokens=10, ignore_eos=True, stop_on_consensus=False)
+    turns = [Turn("A", "Eerste ridder spreekt over de cache.", sp), Turn("B", "Tweede.", sp)]
+    want = [o.ids for o in eng().run_turns(turns)]
+    e = eng()
+    started = e.start_turns(turns)
+    seqs = [s for s, _, _ in started]
+    got = [[f] for _, f, _ in started]
+    for steps in (4, 5):
+        new = e.continue_decode(seqs, turns, [g[-1] for g in got], steps)
+        for g, n in zip(got, new):
+            g.extend(n)
+    assert got == want
+    assert all(s.state_len == s.length for s in seqs)
