@@ -75,7 +75,7 @@ void scalar_norm_add(torch::Tensor res, torch::Tensor y, torch::Tensor g, double
 // conv [n_slots, 2, keep, W] fp32; slots index its first axis
 void chk_conv(const torch::Tensor& conv, const torch::Tensor& w, int64_t W, int64_t sub) {
   chk_f32(conv, "conv"); chk_f32(w, "w");
-  TORCH_CHECK(w.dim() == 2 && w.size(0) == W && w.size(1) >= 1 && w.size(1) <= 8, "conv taps must be 1..8, w [W, taps]");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == W && w.size(1) >= 1 && w.size(1) <= 16, "conv taps must be 1..16, w [W, taps]");
   TORCH_CHECK(conv.dim() == 4 && conv.size(1) == 2 && conv.size(3) == W && conv.size(2) >= std::max<int64_t>(w.size(1) - 1, 1),
               "conv state must be [slots, 2, >= taps - 1, W]");
   TORCH_CHECK(sub == 0 || sub == 1, "sub must be 0 or 1");

@@ -18,7 +18,7 @@ namespace {
 
 using rt::DT;
 constexpr int kThreads = 256;
-constexpr int kMaxTaps = 8;
+constexpr int kMaxTaps = 16;
 
 template <typename IT, typename OT>
 __global__ void __launch_bounds__(1024) scalar_rms_norm_kernel(OT* __restrict__ out, const IT* __restrict__ x,

@@ -489,6 +489,11 @@ class Engine:
         wanted logits [n, vocab] fp32 in entry order. ``end``: keys whose blocks and state are
         given back after the step. Steps made only of single tokens of running sequences take
         the decode launch (split keys), every other step the varlen launch."""
+        entries = [e for e in entries if len(e[1]) > 0]
+        if not entries:                 # nothing to run: only hand back what has ended
+            for key in end:
+                self.release(key)
+            return torch.zeros(0, self.cfg.vocab, dtype=torch.float32)
         with self._on_stream():
             spans = [self.reserve(self.kv.seq(key), toks) for key, toks, _ in entries]
             single = all(len(ids) == 1 and st > 0 for _, st, ids in spans)
