@@ -18,7 +18,6 @@ from theroundtaible_amd.models.config import config_from_dir, get_config
 from theroundtaible_amd.models.weights import layout_for
 
 GPU = pytest.mark.gpu
-DEVICES = ["cpu", pytest.param("cuda:0", marks=GPU)]
 RUNS = [("cpu", "fp32"), pytest.param(("cuda:0", "fp32"), marks=GPU), pytest.param(("cuda:0", "bf16"), marks=GPU)]
 
 

@@ -13,11 +13,17 @@ them in one batch; only the attention launch differs):
     q     = cq @ Wuq^T ; q_lat = q_nope . Wuk   hipBLASLt (batched over heads): the query moves
                                                 into latent space, so keys are the cached rows
     o_lat = latent_attention(q_lat, q_rot)      L3 (HIP): causal, sink in the denominator, all heads
-                                                of a row share each staged key tile
+                                                of a row share each staged key tile (bf16: 32x32x16
+                                                MFMA; fp32 and odd sizes: plain FMA); a decode step
+                                                splits each row's keys over workgroups + a combine
     o     = gate_mul(o_lat . Wuv, proj)         hipBLASLt + L4 (HIP): sigmoid output gate
     x    += scalar_norm(o @ Wo^T)               hipBLASLt + L5 (HIP): post-norm + fp32 residual add
     h     = canon_norm(x)                       L1 (second convolution state)
     x    += scalar_norm(poly_norm(h @ Wup^T) @ Wdown^T)      hipBLASLt + L6 + L5
+
+A decode step (one row per sequence, the launch sequence the captured graph replays) runs the five
+linears on the skinny decode GEMM (shuffled weight copies, ``decode_weights``) and shifts the
+convolution state inside L1; varlen steps use the library GEMMs and a separate state launch.
 
 The residual stream, every norm, the convolution state, positions / angles, scores and softmax
 are fp32 whatever the model dtype; the GEMM operands and the cache take the model dtype.
@@ -43,10 +49,6 @@ class _Rows:
     start_pos: torch.Tensor
     cu_q: torch.Tensor
     slots: torch.Tensor
-
-
-def x_is_cuda(t: torch.Tensor) -> bool:
-    return t.is_cuda
 
 
 class MupulornModel:
@@ -194,7 +196,7 @@ class MupulornModel:
         b = self._rows(positions, meta)
         decode = meta.kind == "decode"
         splits = self.decode_splits(T) if decode else 1
-        skinny = decode and T <= 32 and x_is_cuda(ids) and self.use_skinny and bool(self.decode_weights())
+        skinny = decode and T <= 32 and ids.is_cuda and self.use_skinny and bool(self.decode_weights())
         x = F.embedding(ids, self.w["embed"]).float()
         for l, ls in enumerate(cfg.layers):
             lw, m = self.layers[ls.source], ls.mixer
