@@ -155,13 +155,20 @@ def test_whole_prompt_and_layers(tmp_path, run):
 
 
 @pytest.mark.parametrize("run", RUNS)
-@pytest.mark.parametrize("shape", ["one-head", "wide", "taps1", "no-rot-tail"])
+@pytest.mark.parametrize("shape", ["one-head", "wide", "taps1", "no-rot-tail", "tiles"])
 def test_other_sizes(tmp_path, run, shape):
     """Sizes that the usual test model makes equal or 1: a single head, rows wider than a key
     tile's lanes, one tap (no state), rotation on a part of the rotary entries only."""
     lay = {"one-head": [{"type": "latent_attention", "mixer": mixer(1, 16, 4, 8, 16, 8), "mlp": {"kind": "dense", "ff": 24}}],
            "wide": [{"type": "latent_attention", "mixer": mixer(5, 24, 10, 12, 136, 36), "mlp": None},
                     {"type": "latent_attention", "mixer": mixer(9, 8, 2, 8, 72, 16), "mlp": {"kind": "dense", "ff": 200}}],
+           # latents of 64 and 128 with rotary parts of 16 and 32 (the shapes the bf16 matrix-core
+           # attention takes) beside one it does not take, and a layer that shares the first one's weights
+           "tiles": [{"type": "latent_attention", "mixer": mixer(4, 32, 16, 24, 64, 48), "mlp": {"kind": "dense", "ff": 72}},
+                     {"type": "latent_attention", "mixer": mixer(6, 16, 32, 16, 128, 40, base=300.0), "mlp": None},
+                     {"type": "latent_attention", "mixer": mixer(3, 16, 8, 16, 96, 24), "mlp": {"kind": "dense", "ff": 40}},
+                     {"type": "latent_attention", "mixer": mixer(4, 32, 16, 24, 64, 48), "mlp": {"kind": "dense", "ff": 72},
+                      "weights_of": 0}],
            "taps1": None, "no-rot-tail": [{"type": "latent_attention", "mixer": mixer(2, 6, 7, 5, 18, 10, rot_dims=2),
                                            "mlp": {"kind": "dense", "ff": 30}}]}[shape]
     cfg = make_config(width=40, vocab=61, taps=1 if shape == "taps1" else 3, layers=lay, logit_scale=1.0, softcap=8.0)
