@@ -200,12 +200,13 @@ ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": pars
 
 PRESETS.update({
     # Mupulorn (latent attention + input convolutions + PolyNorm feed-forward), random-init sizes:
-    # a test-sized stack and two whose layers have the shapes of 1B / 8B-class models
+    # a test-sized stack and three whose layers have the shapes of 1B / 3B / 8B-class models
     "tiny-mupulorn": mupulorn_config("tiny-mupulorn", 3, 128, 4, 32, 16, 32, 64, 48, 256, 32000, taps=4,
                                      shared_every=2),
     # (the two-matrix feed-forward is 1.5x as wide as the gated three-matrix one of the Llama preset
     # of the same class, so a layer holds about the same weights)
     "mupulorn-1b": mupulorn_config("mupulorn-1b", 16, 2048, 16, 128, 64, 128, 512, 768, 12288, 128256),
+    "mupulorn-3b": mupulorn_config("mupulorn-3b", 28, 3072, 24, 128, 64, 128, 256, 1024, 12288, 128256),
     "mupulorn-8b": mupulorn_config("mupulorn-8b", 32, 4096, 32, 128, 64, 128, 512, 1536, 21504, 128256),
 })
 
