@@ -385,3 +385,31 @@ def test_serving_entry_points_match_run_turns():
             g.extend(n)
     assert got == want
     assert all(s.state_len == s.length for s in seqs)
+
+
+def test_latent_cache_slots_rollback_and_fork():
+    """The cache manager alone: slots are handed out on first use and come back with the sequence;
+    a roll-back keeps a stateful sequence only at its state's exact length; a fork copies the state."""
+    from theroundtaible_amd.engine.kv_cache import LatentKVCache
+    kv = LatentKVCache([10, 6], conv_width=4, taps=3, num_blocks=8, block_size=4, device="cpu",
+                       dtype=torch.float32, n_slots=2)
+    a = kv.seq("a")
+    kv.ensure_capacity(a, 6)
+    a.tokens.extend(range(6))
+    assert kv.slot_of(a) == 0 and kv.slot_of(a) == 0
+    a.state_len = 6
+    kv.conv[1][a.slot].fill_(3.0)
+    b = kv.fork("a", "b")                       # shares pages, owns a copy of the state
+    assert b.slot == 1 and b.state_len == 6 and float(kv.conv[1][b.slot].mean()) == 3.0
+    with pytest.raises(KVCacheOOM):
+        kv.slot_of(kv.seq("c"))                 # both slots are taken
+    kv.truncate(a, 6)                           # the state's own length: kept
+    assert a.length == 6
+    kv.truncate(a, 4)                           # anything else: the sequence starts over
+    assert a.length == 0 and a.state_len == 0 and a.blocks == []
+    kv.free_seq("b")
+    assert kv.slot_of(kv.seq("c")) == 1         # b's slot is used again
+    kv.free_seq("a")
+    kv.free_seq("c")
+    assert kv.alloc.num_free == 8 and sorted(kv.state.free) == [0, 1]
+    assert kv.layer_rows(0).shape == (8, 4, 10) and kv.layer_rows(1).shape == (8, 4, 6)
