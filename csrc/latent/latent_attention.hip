@@ -260,6 +260,10 @@ __global__ void __launch_bounds__(256) latent_combine_kernel(OT* __restrict__ ou
 typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+#ifndef RT_STAGE_BATCH
+#define RT_STAGE_BATCH 9
+#endif
+constexpr int kStageBatch = RT_STAGE_BATCH;   // staging loads in flight per lane
 constexpr int kVRow = KT * 2 + 16;   // bytes per V^T / P row in LDS (64 keys + pad)
 
 RT_DEVICE int swap23(int x) { return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1); }
@@ -333,9 +337,8 @@ __global__ void __launch_bounds__(kThreads) latent_attn_mfma_kernel(AttnArgs a) 
       const int kp = k0 + lane;
       const bool ok = kp < ke;
       const uint16_t* src = cache + ((size_t)(ok ? bt[kp / a.BS] : 0) * a.BS + (ok ? kp % a.BS : 0)) * Dk;
-      for (int ch = wave; ch < nch; ch += kWaves) {
-        rt::u32x4 v = {0u, 0u, 0u, 0u};
-        if (ok) v = *reinterpret_cast<const rt::u32x4*>(src + ch * 8);
+      // a batch of chunk loads is issued before the first is consumed
+      auto put = [&](int ch, const rt::u32x4& v) {
         *reinterpret_cast<rt::u32x4*>(Kt + (size_t)lane * krow_b + ch * 16) = v;
         if (ch * 8 < C) {
           uint16_t* vt = reinterpret_cast<uint16_t*>(Vt + (size_t)(ch * 8) * kVRow) + lane;
@@ -344,6 +347,20 @@ __global__ void __launch_bounds__(kThreads) latent_attn_mfma_kernel(AttnArgs a) 
             vt[(size_t)(2 * j) * (kVRow / 2)] = (uint16_t)(v[j] & 0xffffu);
             vt[(size_t)(2 * j + 1) * (kVRow / 2)] = (uint16_t)(v[j] >> 16);
           }
+        }
+      };
+      for (int ch = wave; ch < nch; ch += kStageBatch * kWaves) {
+        rt::u32x4 v[kStageBatch];
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+          v[u] = rt::u32x4{0u, 0u, 0u, 0u};
+          const int cu_ = ch + u * kWaves;
+          if (ok && cu_ < nch) v[u] = *reinterpret_cast<const rt::u32x4*>(src + cu_ * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+          const int cu_ = ch + u * kWaves;
+          if (cu_ < nch) put(cu_, v[u]);
         }
       }
     }
