@@ -195,7 +195,49 @@ class StateSlots:
         self.free.append(slot)
 
 
-class LatentKVCache(PagedKVCache):
+class StatefulPagedCache(PagedKVCache):
+    """A paged cache whose sequences also keep a running state in a slot of a fixed pool
+    (``self.state``: :class:`StateSlots`). ``state_tensors()`` lists every tensor indexed by slot on
+    its first axis. The state belongs to exactly ``state_len`` tokens of its sequence: rolling a
+    sequence back to any other length drops it, and the sequence restarts from position 0."""
+
+    state: StateSlots
+
+    def state_tensors(self) -> List[torch.Tensor]:
+        raise NotImplementedError
+
+    def slot_of(self, s: SeqState) -> int:
+        """The sequence's state slot (taken on first use)."""
+        if s.slot is None:
+            s.slot = self.state.take()
+            s.state_len = 0
+        return s.slot
+
+    def _state_rollback(self, s: SeqState, n_tokens: int) -> int:
+        if n_tokens == s.state_len or s.slot is None:
+            return n_tokens
+        s.state_len = 0         # the convolution inputs ahead of `n_tokens` are gone: start over
+        return 0
+
+    def _release_state(self, s: SeqState) -> None:
+        if s.slot is not None:
+            self.state.give(s.slot)
+            s.slot = None
+
+    def fork(self, src: str, dst: str, copy: bool = False) -> SeqState:
+        b = super().fork(src, dst, copy=copy)
+        a = self.seqs[src]
+        if a.slot is not None and a.state_len == a.length:
+            b.slot = self.state.take()
+            b.state_len = a.state_len
+            for c in self.state_tensors():
+                c[b.slot].copy_(c[a.slot])
+        else:
+            self.truncate(b, 0)
+        return b
+
+
+class LatentKVCache(StatefulPagedCache):
     """Paged cache of latent-attention layers plus the input-convolution states.
 
     Per layer ``l`` one tensor ``rows[l]`` ``[num_blocks, block_size, row_l]``: token ``t`` of a
@@ -243,32 +285,56 @@ class LatentKVCache(PagedKVCache):
         for r in self.rows:
             r.index_copy_(0, di, r.index_select(0, si))
 
-    def slot_of(self, s: SeqState) -> int:
-        """The sequence's state slot (taken on first use)."""
-        if s.slot is None:
-            s.slot = self.state.take()
-            s.state_len = 0
-        return s.slot
+    def state_tensors(self) -> List[torch.Tensor]:
+        return self.conv
 
-    def _state_rollback(self, s: SeqState, n_tokens: int) -> int:
-        if n_tokens == s.state_len or s.slot is None:
-            return n_tokens
-        s.state_len = 0         # the convolution inputs ahead of `n_tokens` are gone: start over
-        return 0
 
-    def _release_state(self, s: SeqState) -> None:
-        if s.slot is not None:
-            self.state.give(s.slot)
-            s.slot = None
+class GroupedKVCache(StatefulPagedCache):
+    """Paged keys and values of grouped-attention layers whose shapes differ from layer to layer,
+    plus per-sequence running states.
 
-    def fork(self, src: str, dst: str, copy: bool = False) -> SeqState:
-        b = super().fork(src, dst, copy=copy)
-        a = self.seqs[src]
-        if a.slot is not None and a.state_len == a.length:
-            b.slot = self.state.take()
-            b.state_len = a.state_len
-            for c in self.conv:
-                c[b.slot].copy_(c[a.slot])
-        else:
-            self.truncate(b, 0)
-        return b
+    Layer run ``l``: ``k[l]`` ``[num_blocks, kv_heads_l, block_size, dim_l]`` and ``v[l]``
+    ``[num_blocks, kv_heads_l, block_size, vdim_l]``; token ``t`` of a sequence lives at
+    ``block_tables[t // block_size]``, offset ``t % block_size``. ``shapes`` gives
+    ``(kv_heads, dim, vdim)`` per run.
+
+    States, fp32, one row per slot: ``shift[l]`` ``[n_slots, width]`` is the previous token's
+    normed mixer input (token shift); ``rec[l]`` ``[n_slots, rec_width_l]`` the state of the
+    layer's recurrence (None for a layer without one). A sequence at position 0 never reads its
+    slot, so a reused slot needs no clearing."""
+
+    def __init__(self, shapes, width: int, rec_widths, num_blocks: int, block_size: int, device,
+                 dtype=torch.bfloat16, n_slots: int = 16):
+        self.n_layers = len(shapes)
+        self.shapes = [tuple(int(x) for x in sh) for sh in shapes]
+        self.n_kv_heads = max(sh[0] for sh in self.shapes)
+        self.head_dim = max(max(sh[1], sh[2]) for sh in self.shapes)
+        self.block_size, self.num_blocks = block_size, num_blocks
+        self.device, self.dtype = device, dtype
+        # zero-init: tail rows of a partial block are masked, never skipped, so they must be finite
+        self.k = [torch.zeros(num_blocks, g, block_size, dk, dtype=dtype, device=device) for g, dk, _ in self.shapes]
+        self.v = [torch.zeros(num_blocks, g, block_size, dv, dtype=dtype, device=device) for g, _, dv in self.shapes]
+        self.alloc = BlockAllocator(num_blocks)
+        self.seqs = {}
+        self.state = StateSlots(n_slots)
+        self.shift = [torch.zeros(n_slots, width, dtype=torch.float32, device=device) for _ in self.shapes]
+        self.rec = [torch.zeros(n_slots, w, dtype=torch.float32, device=device) if w else None for w in rec_widths]
+
+    @staticmethod
+    def bytes_per_block(shapes, block_size, dtype_bytes=2) -> int:   # type: ignore[override]
+        return sum(g * (dk + dv) for g, dk, dv in shapes) * block_size * dtype_bytes
+
+    def k_layer(self, l: int) -> torch.Tensor:
+        return self.k[l]
+
+    def v_layer(self, l: int) -> torch.Tensor:
+        return self.v[l]
+
+    def copy_blocks(self, src: List[int], dst: List[int]) -> None:
+        si = torch.tensor(src, dtype=torch.int64, device=self.device)
+        di = torch.tensor(dst, dtype=torch.int64, device=self.device)
+        for t in self.k + self.v:
+            t.index_copy_(0, di, t.index_select(0, si))
+
+    def state_tensors(self) -> List[torch.Tensor]:
+        return self.shift + [r for r in self.rec if r is not None]

@@ -28,14 +28,70 @@ class LatentAttentionSpec:
 
 
 @dataclass(frozen=True)
+class RotarySpec:
+    """Rotary positions on the leading ``dims`` entries of a head, entry 2i paired with 2i + 1:
+    angle = position * base^(-2i / dims), frequencies optionally rescaled (``scaling`` as in
+    ``ModelConfig.rope_scaling``, e.g. ("llama3", factor, low, high, original))."""
+    base: float
+    dims: int
+    scaling: Optional[tuple] = None
+
+
+@dataclass(frozen=True)
+class GroupedAttentionSpec:
+    """Causal attention with ``heads`` query heads over ``kv_heads`` key / value heads (query head
+    h reads key / value head h // (heads / kv_heads)); queries and keys are divided by their root
+    mean square per head (after the rotation, if any). ``sink`` is a constant added to the softmax
+    denominator as exp(0) * sink: a key of score 0 without a value (0 = ordinary softmax).
+    ``head_temp``: every head multiplies its scores by a learned number (tensor ``temp``).
+    ``value_from_key``: there is no value projection, the values are the projected keys as they
+    are before the norm."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: Optional[RotarySpec] = None
+    sink: float = 0.0
+    head_temp: bool = False
+    value_from_key: bool = False
+
+    @property
+    def group(self) -> int:
+        return self.heads // self.kv_heads
+
+    @property
+    def cache_row(self) -> int:
+        """Cached numbers per token: keys and values of every key / value head."""
+        return self.kv_heads * (self.dim + self.vdim)
+
+
+@dataclass(frozen=True)
+class MinGRUSpec:
+    """Gated recurrence whose gates read only the current token (minGRU), ``width`` channels:
+    S_t = (1 - z_t) S_(t-1) + z_t c_t, output gated by silu of a third projection."""
+    width: int
+
+
+@dataclass(frozen=True)
+class ParallelSpec:
+    """Two mixers reading the same input: attention (``left``) and a minGRU (``right``); the layer
+    adds half the sum of their RMS-normed outputs."""
+    left: GroupedAttentionSpec
+    right: MinGRUSpec
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One decoder layer of a per-layer-configured model: its mixer, its feed-forward (``ff`` 0 =
-    none) and ``source``, the layer whose tensors it uses (itself unless its weights are shared)."""
+    none) and ``source``, the layer whose tensors it uses (itself unless its weights are shared).
+    ``ff_limit``: the clamp of a limited gated feed-forward."""
     mixer_type: str
-    mixer: LatentAttentionSpec
+    mixer: object
     ff: int
     ff_kind: str
     source: int
+    ff_limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -63,6 +119,7 @@ class ModelConfig:
     canon_taps: int = 0
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
+    embed_scale: float = 1.0      # the embedding row is multiplied by it ("goganex")
 
     @property
     def q_size(self) -> int:
@@ -78,6 +135,15 @@ class ModelConfig:
 
     def n_params(self) -> int:
         h, f, v, L = self.hidden, self.ffn, self.vocab, self.n_layers
+        if self.arch == "goganex":
+            from .weights import goganex_layout
+            n = 0
+            for shape, _, _ in goganex_layout(self).values():
+                k = 1
+                for d in shape:
+                    k *= d
+                n += k
+            return n
         if self.layers is not None:
             n = 2 * v * h + 1
             for i, ls in enumerate(self.layers):
@@ -101,7 +167,7 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.layers is not None:
-            return sum(ls.mixer.cache_row for ls in self.layers) * dtype_bytes
+            return sum(attention_of(ls).cache_row for ls in self.layers) * dtype_bytes
         return 2 * self.n_layers * self.n_kv_heads * self.head_dim * dtype_bytes
 
 
@@ -174,6 +240,87 @@ def parse_mupulorn(d: dict, name: str = "mupulorn") -> ModelConfig:
                        logit_softcap=float(d["logit_softcap"]))
 
 
+def attention_of(ls: LayerSpec):
+    """The attention part of a layer's mixer (the left half of a parallel mixer)."""
+    return ls.mixer.left if isinstance(ls.mixer, ParallelSpec) else ls.mixer
+
+
+def _grouped_attention(mx: dict, where: str, **kind) -> GroupedAttentionSpec:
+    rot = None
+    if mx.get("rot") is not None:
+        r = mx["rot"]
+        sc = r.get("scaling")
+        rot = RotarySpec(float(r["base"]), int(r["dims"]),
+                         ("llama3", float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
+                         if sc is not None else None)
+    a = GroupedAttentionSpec(int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]), int(mx["vdim"]), float(mx["scale"]),
+                             rot, **kind)
+    if a.heads % a.kv_heads:
+        raise ValueError(f"{where}: {a.heads} query heads do not divide over {a.kv_heads} key/value heads")
+    if rot is not None and (rot.dims > a.dim or rot.dims % 2):
+        raise ValueError(f"{where}: rot.dims {rot.dims} does not fit dim {a.dim}")
+    if a.value_from_key and a.vdim != a.dim:
+        raise ValueError(f"{where}: values are the keys, so vdim {a.vdim} must equal dim {a.dim}")
+    return a
+
+
+def parse_goganex(d: dict, name: str = "goganex") -> ModelConfig:
+    """``config.json`` of a Goganex checkpoint -> :class:`ModelConfig`. ``layers`` of the result
+    are the layer RUNS in execution order: the checkpoint layers ``loop.start .. loop.stop - 1``
+    are run ``loop.times`` times in a row with the same tensors (``LayerSpec.source``), every run
+    with a cache and state of its own."""
+    raw = d["layers"]
+    order = list(range(len(raw)))
+    lp = d.get("loop")
+    if lp is not None:
+        a, b, n = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+        if not (0 <= a <= b <= len(raw)) or n < 1:
+            raise ValueError(f"{name}: loop {lp} does not fit {len(raw)} layers")
+        order = order[:a] + order[a:b] * n + order[b:]
+    specs = []
+    for i in order:
+        e, where = raw[i], f"{name}: layer {i}"
+        if e["type"] == "attention":
+            mixer = _grouped_attention(e["mixer"], where, sink=1.0, head_temp=True)
+        elif e["type"] == "parallel":
+            mixer = ParallelSpec(_grouped_attention(e["mixer"]["left"], where, value_from_key=True),
+                                 MinGRUSpec(int(e["mixer"]["right"]["width"])))
+        else:
+            raise ValueError(f"{where}: unknown mixer type '{e['type']}'")
+        mlp = e.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"{where}: unknown feed-forward kind '{mlp['kind']}'")
+        specs.append(LayerSpec(e["type"], mixer, int(mlp["ff"]) if mlp is not None else 0, "dense", i,
+                               float(mlp["limit"]) if mlp is not None else 0.0))
+    top = max((attention_of(s) for s in specs), key=lambda m: m.heads)
+    rots = [attention_of(s).rot for s in specs if attention_of(s).rot is not None]
+    return ModelConfig(name, "goganex", len(specs), int(d["width"]), top.heads, top.kv_heads, top.dim,
+                       max(s.ff for s in specs), int(d["vocab"]), int(d.get("max_pos", 1 << 17)),
+                       rots[0].base if rots else 0.0, float(d["norm"]["eps"]), layers=tuple(specs),
+                       embed_scale=float(d.get("embedding", {}).get("scale", 1.0)))
+
+
+def goganex_config(name: str, n_layers: int, width: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                   parallel_every: int = 4, gru_width: int = 0, loop: Optional[Tuple[int, int, int]] = None,
+                   rot_base: float = 500000.0, limit: float = 7.0, max_pos: int = 1 << 17) -> ModelConfig:
+    """A Goganex stack from a few sizes (benchmarks and presets): attention layers with every
+    ``parallel_every``-th layer a parallel attention + minGRU layer (0: none)."""
+    att = {"type": "attention",
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 1.5 * dim ** -0.5,
+                     "rot": {"base": rot_base, "dims": dim, "scaling": None}},
+           "mlp": {"kind": "dense", "ff": ff, "limit": limit} if ff else None}
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5},
+                     "right": {"width": gru_width or width}},
+           "mlp": att["mlp"]}
+    layers = [par if parallel_every and (i + 1) % parallel_every == 0 else att for i in range(n_layers)]
+    d = {"architecture": "Goganex", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5},
+         "vocab": vocab, "width": width, "max_pos": max_pos}
+    if loop is not None:
+        d["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return parse_goganex(d, name)
+
+
 def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
                     kv_rank: int, q_rank: int, ff: int, vocab: int, taps: int = 4, shared_every: int = 0,
                     rot_base: float = 10000.0, max_pos: int = 1 << 17) -> ModelConfig:
@@ -196,7 +343,7 @@ def mupulorn_config(name: str, n_layers: int, width: int, heads: int, dim: int, 
 
 
 # config.json "architecture" -> parser (checkpoint directories name their own model class)
-ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": parse_mupulorn}
+ARCHITECTURES: Dict[str, Callable[[dict, str], ModelConfig]] = {"Mupulorn": parse_mupulorn, "Goganex": parse_goganex}
 
 PRESETS.update({
     # Mupulorn (latent attention + input convolutions + PolyNorm feed-forward), random-init sizes:
@@ -208,6 +355,18 @@ PRESETS.update({
     "mupulorn-1b": mupulorn_config("mupulorn-1b", 16, 2048, 16, 128, 64, 128, 512, 768, 12288, 128256),
     "mupulorn-3b": mupulorn_config("mupulorn-3b", 28, 3072, 24, 128, 64, 128, 256, 1024, 12288, 128256),
     "mupulorn-8b": mupulorn_config("mupulorn-8b", 32, 4096, 32, 128, 64, 128, 512, 1536, 21504, 128256),
+})
+
+
+PRESETS.update({
+    # Goganex (grouped attention with a softmax sink, token shift, parallel attention + minGRU
+    # layers, clamped gated feed-forward), random-init sizes: a test-sized stack with a looped
+    # middle, and stacks whose layers have the shapes of 1B / 3B / 8B-class Llama models
+    "tiny-goganex": goganex_config("tiny-goganex", 3, 128, 4, 2, 32, 256, 32000, parallel_every=3, gru_width=96,
+                                   loop=(1, 3, 2)),
+    "goganex-1b": goganex_config("goganex-1b", 16, 2048, 32, 8, 64, 8192, 128256),
+    "goganex-3b": goganex_config("goganex-3b", 28, 3072, 24, 8, 128, 8192, 128256),
+    "goganex-8b": goganex_config("goganex-8b", 32, 4096, 32, 8, 128, 14336, 128256),
 })
 
 

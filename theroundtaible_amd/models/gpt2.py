@@ -89,5 +89,8 @@ def build_model(cfg: ModelConfig, weights, device, dtype=torch.bfloat16, tp: Opt
     if cfg.arch == "mupulorn":
         from .mupulorn import MupulornModel
         return MupulornModel(cfg, weights, device, dtype, tp)
+    if cfg.arch == "goganex":
+        from .goganex import GoganexModel
+        return GoganexModel(cfg, weights, device, dtype, tp)
     from .llama import LlamaModel
     return LlamaModel(cfg, weights, device, dtype, tp)

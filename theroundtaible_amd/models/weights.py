@@ -108,9 +108,55 @@ def mupulorn_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, O
     return lay
 
 
+def goganex_layout(cfg: ModelConfig) -> Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]]:
+    """Checkpoint names and shapes of a Goganex model (linear weights [out, in]). A looped layer
+    has one set of tensors, named by its place in the checkpoint's layer list. Not
+    tensor-parallel: every kind is None."""
+    from .config import ParallelSpec
+    W = cfg.hidden
+    lay: Dict[str, Tuple[Tuple[int, ...], str, Optional[str]]] = {
+        "embed": ((cfg.vocab, W), "normal", None),
+        "final.norm": ((W,), "ones", None),
+        "head": ((cfg.vocab, W), "normal", None),
+    }
+    for ls in cfg.layers:
+        p = f"l{ls.source}."
+        if p + "norm1" in lay:
+            continue
+        lay[p + "norm1"] = ((W,), "ones", None)
+        lay[p + "shift"] = ((W,), "half", None)
+        if isinstance(ls.mixer, ParallelSpec):
+            a, r = ls.mixer.left, ls.mixer.right
+            lay[p + "mix.left.q"] = ((a.heads * a.dim, W), "normal", None)
+            lay[p + "mix.left.k"] = ((a.kv_heads * a.dim, W), "normal", None)
+            lay[p + "mix.left.o"] = ((W, a.heads * a.vdim), "normal", None)
+            for n in ("z", "x", "g"):
+                lay[p + f"mix.right.{n}"] = ((r.width, W), "normal", None)
+            lay[p + "mix.right.z.b"] = ((r.width,), "zeros", None)
+            lay[p + "mix.right.x.b"] = ((r.width,), "zeros", None)
+            lay[p + "mix.right.o"] = ((W, r.width), "normal", None)
+            lay[p + "mix.left.out"] = ((W,), "ones", None)
+            lay[p + "mix.right.out"] = ((W,), "ones", None)
+        else:
+            a = ls.mixer
+            lay[p + "mix.q"] = ((a.heads * a.dim, W), "normal", None)
+            lay[p + "mix.k"] = ((a.kv_heads * a.dim, W), "normal", None)
+            lay[p + "mix.v"] = ((a.kv_heads * a.vdim, W), "normal", None)
+            lay[p + "mix.temp"] = ((a.heads,), "ones", None)
+            lay[p + "mix.o"] = ((W, a.heads * a.vdim), "normal", None)
+        if ls.ff:
+            lay[p + "norm2"] = ((W,), "ones", None)
+            lay[p + "mlp.gate"] = ((ls.ff, W), "normal", None)
+            lay[p + "mlp.up"] = ((ls.ff, W), "normal", None)
+            lay[p + "mlp.down"] = ((W, ls.ff), "normal", None)
+    return lay
+
+
 def layout_for(cfg: ModelConfig):
     if cfg.arch == "mupulorn":
         return mupulorn_layout(cfg)
+    if cfg.arch == "goganex":
+        return goganex_layout(cfg)
     return gpt2_layout(cfg) if cfg.arch == "gpt2" else llama_layout(cfg)
 
 
@@ -190,6 +236,8 @@ def _init(shape, init, std, g, device, dtype):
         return torch.ones(shape, device=device, dtype=dtype)
     if init == "zeros":
         return torch.zeros(shape, device=device, dtype=dtype)
+    if init == "half":      # token-shift mixing weights
+        return torch.full(shape, 0.5, device=device, dtype=dtype)
     if init == "poly":      # PolyNorm coefficients: equal thirds, no offset
         return torch.tensor([1 / 3, 1 / 3, 1 / 3, 0.0], device=device, dtype=dtype)
     if init == "small":     # input-convolution taps
@@ -262,10 +310,10 @@ def load_safetensors(cfg: ModelConfig, path: str, device, dtype, tp: TPInfo) -> 
         tensors.update(load_file(f, device="cpu"))
     lay = layout_for(cfg)
     out = {}
-    if cfg.arch == "mupulorn":
+    if cfg.arch in ("mupulorn", "goganex"):
         # the checkpoint's own names; integer tables keep their type, everything else takes `dtype`
         if tp.size > 1:
-            raise ValueError("mupulorn checkpoints are not tensor-parallel")
+            raise ValueError(f"{cfg.arch} checkpoints are not tensor-parallel")
         for name, (shape, _, _) in lay.items():
             if name not in tensors:
                 raise KeyError(f"{path}: tensor '{name}' is missing")

@@ -1,0 +1,332 @@
+"""Ops of decoders that mix grouped attention with recurrent layers: token shift fused with the
+RMS norm ahead of a mixer, query / key preparation (rotary pairs, per-head unit RMS) with the paged
+cache write, grouped-query attention with an optional softmax sink and per-head temperature, the
+minGRU scan, the two-branch normed residual add, residual add + RMS norm, and the clamped gated
+feed-forward activation.
+
+GPU tensors go to the HIP kernels of ``theroundtaible_amd._C_hybrid`` (``csrc/hybrid/``, built
+in-tree by ``csrc/build.py``; :func:`ensure_built` compiles it on first use in a fresh checkout);
+CPU tensors run the PyTorch statements at the end of this file. There is no silent fallback on a
+GPU.
+
+Every kernel computes in fp32 and reads / writes bf16 or fp32 tensors as given; the residual
+stream and every running state are always fp32.
+"""
+from __future__ import annotations
+
+import os
+import sys
+from typing import Optional, Tuple
+
+import torch
+
+_NATIVE = None
+_NATIVE_ERR: Optional[BaseException] = None
+
+MAX_HEAD_DIM = 256       # widest query / key / value head the kernels hold in registers
+PAIRS_PER_TILE = 32      # (query row, head) pairs one attention workgroup takes
+
+
+def native():
+    global _NATIVE, _NATIVE_ERR
+    if _NATIVE is None and _NATIVE_ERR is None:
+        try:
+            from .. import _C_hybrid  # type: ignore
+            _NATIVE = _C_hybrid
+        except BaseException as e:  # noqa: BLE001
+            _NATIVE_ERR = e
+    if _NATIVE is None:
+        raise RuntimeError(f"theroundtaible_amd._C_hybrid (HIP kernels) is not built/importable: {_NATIVE_ERR}. "
+                           f"Run `python csrc/build.py hybrid` (or __graft_entry__.build()).")
+    return _NATIVE
+
+
+def ensure_built(verbose: bool = False) -> None:
+    """Compile the extension if it is missing or older than its sources (a fresh checkout's first
+    GPU run); only this family's kernels are compiled."""
+    global _NATIVE_ERR
+    root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    sys.path.insert(0, os.path.join(root, "csrc"))
+    try:
+        import build as csrc_build
+        csrc_build.build_hybrid(verbose=verbose)
+    finally:
+        sys.path.pop(0)
+    _NATIVE_ERR = None
+
+
+def _gpu(t: torch.Tensor) -> bool:
+    return t.is_cuda
+
+
+# ---- token shift + norm ---------------------------------------------------------------------------
+
+def shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype,
+               shift_state: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``x`` [T, W] fp32 residual, ``y`` an optional pending branch output still to be added.
+    With ``xs = x + y`` and ``h_r = xs_r / rms(xs_r) * w``: returns ``(h_r + (p_r - h_r) * mu, xs)``
+    where ``p_r`` is the previous token's ``h``: row r - 1 inside a span, ``state[slot]`` for the
+    first row of a span that continues a sequence, zeros at position 0. ``xs`` is a new tensor
+    when ``y`` is given (other rows of the launch still read the old ``x``), else ``x`` itself.
+    ``shift_state`` (only with ONE row per sequence, a decode step): the same launch also stores
+    ``h_r`` as the sequence's new state, so no :func:`shift_state_update` follows."""
+    if _gpu(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        xs = torch.empty_like(x) if y is not None else x
+        native().shift_norm(out, xs, x, y, w, float(eps), mu, state, row_seq, positions, start_pos, slots,
+                            bool(shift_state))
+        return out, xs
+    return ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state)
+
+
+def shift_state_update(x, w, eps, state, cu_q, slots) -> None:
+    """Store the normed last row of every span as its sequence's state. Runs AFTER
+    :func:`shift_norm` of the same layer (it overwrites what that one reads)."""
+    if _gpu(x):
+        native().shift_state_update(x, w, float(eps), state, cu_q, slots)
+        return
+    ref_shift_state_update(x, w, eps, state, cu_q, slots)
+
+
+# ---- queries, keys, values ------------------------------------------------------------------------
+
+def rotary_table(rot, device) -> Optional[torch.Tensor]:
+    """fp32 frequencies [dims / 2] of a :class:`RotarySpec` (None: no rotation)."""
+    if rot is None or rot.dims == 0:
+        return None
+    from .reference import rope_inv_freq
+    inv, _ = rope_inv_freq(rot.dims, rot.base, rot.scaling)
+    return inv.to(torch.float32).to(device).contiguous()
+
+
+def qk_prep(proj, spec, q_off: int, k_off: int, v_off: int, inv_freq, eps, positions, k_cache, v_cache,
+            slot_mapping, out_dtype) -> torch.Tensor:
+    """``proj`` [T, N]: columns ``q_off ..`` hold the projected queries (heads x dim), ``k_off ..``
+    the keys (kv_heads x dim), ``v_off ..`` the values (kv_heads x vdim; ignored when the values
+    are the keys). Rotates the leading ``2 * len(inv_freq)`` entries of every query / key head
+    (entry 2i with 2i + 1, angle = position * inv_freq[i], fp32), divides each head by its root
+    mean square, writes keys and values to the paged cache at ``slot_mapping`` and returns the
+    queries [T, heads, dim]."""
+    if _gpu(proj):
+        T = proj.shape[0]
+        q = torch.empty(T, spec.heads, spec.dim, dtype=out_dtype, device=proj.device)
+        native().qk_prep(q, proj, int(q_off), int(k_off), int(v_off), bool(spec.value_from_key), inv_freq, float(eps),
+                         positions, k_cache, v_cache, slot_mapping)
+        return q
+    return ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping,
+                       out_dtype)
+
+
+def rows_per_tile(group: int) -> int:
+    """Query rows one varlen attention workgroup takes (its (row, head) pairs share a key tile)."""
+    return max(1, PAIRS_PER_TILE // max(1, group))
+
+
+def tile_map(cu_q: torch.Tensor, start_pos: torch.Tensor, rows: int) -> torch.Tensor:
+    """[n_tiles, 2] int32 (sequence, first row) of the varlen attention launch, heaviest first."""
+    items = []
+    cq, sp = cu_q.tolist(), start_pos.tolist()
+    for s in range(len(sp)):
+        for r in range(cq[s], cq[s + 1], rows):
+            items.append((sp[s] + min(r + rows, cq[s + 1]) - cq[s], s, r))
+    items.sort(key=lambda x: -x[0])
+    return torch.tensor([(s, r) for _, s, r in items], dtype=torch.int32).reshape(-1, 2)
+
+
+class SplitWorkspace:
+    """Split-key scratch of the one-row-per-sequence (decode) attention launch: per (row, head,
+    split) a partial output, running maximum and sum; static, so captured graphs can hold it."""
+
+    def __init__(self, max_rows: int, heads: int, vdim: int, max_splits: int, device):
+        self.max_rows, self.max_splits = max_rows, max_splits
+        self.part_o = torch.empty(max_rows * heads * max_splits * vdim, dtype=torch.float32, device=device)
+        self.part_ml = torch.empty(max_rows * heads * max_splits * 2, dtype=torch.float32, device=device)
+
+
+def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: float, temp=None, sink: float = 0.0,
+                  tiles=None, num_splits: int = 1, workspace: Optional[SplitWorkspace] = None,
+                  out_dtype=None) -> torch.Tensor:
+    """Causal attention of the rows ``q`` [T, H, Dk] (span s = rows ``cu_q[s] .. cu_q[s + 1]`` at
+    positions ``start_pos[s] ..`` of sequence s) over the paged keys ``k_cache`` [nb, G, BS, Dk]
+    and values ``v_cache`` [nb, G, BS, Dv]: score = q . k * scale (* ``temp[h]``), weights
+    exp(s_j) / (``sink`` + sum exp(s_j)). Returns [T, H * Dv]. ``tiles``: :func:`tile_map` on the
+    device; ``num_splits`` > 1 (one row per span: a decode step) cuts every row's keys into that
+    many ranges merged by a second launch."""
+    out_dtype = out_dtype or q.dtype
+    if _gpu(q):
+        T, H, _ = q.shape
+        G, Dv = k_cache.shape[1], v_cache.shape[3]
+        out = torch.empty(T, H * Dv, dtype=out_dtype, device=q.device)
+        rows = 1 if num_splits > 1 else rows_per_tile(H // G)
+        if tiles is None:
+            tiles = tile_map(cu_q.cpu(), start_pos.cpu(), rows).to(q.device)
+        if num_splits > 1 and workspace is None:
+            workspace = SplitWorkspace(T, H, Dv, num_splits, q.device)
+        native().gqa_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tiles, temp, float(scale),
+                               float(sink), rows, int(num_splits),
+                               workspace.part_o if num_splits > 1 else None,
+                               workspace.part_ml if num_splits > 1 else None)
+        return out
+    return ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype)
+
+
+# ---- minGRU ---------------------------------------------------------------------------------------
+
+def mingru_scan(proj, z_off: int, x_off: int, g_off: int, width: int, bz, bx, state, cu_q, start_pos, slots,
+                out_dtype) -> torch.Tensor:
+    """``proj`` [T, N] holds the three projections of the recurrence at the given column offsets.
+    z = sigmoid(p_z + bz); u = p_x + bx; c = u + 1/2 where u >= 0, sigmoid(u) below;
+    S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, from ``state[slot]`` (zeros at position 0);
+    returns S_t * silu(p_g) [T, width] and leaves every span's last S in ``state``. fp32 inside."""
+    if _gpu(proj):
+        out = torch.empty(proj.shape[0], width, dtype=out_dtype, device=proj.device)
+        native().mingru_scan(out, proj, int(z_off), int(x_off), int(g_off), bz, bx, state, cu_q, start_pos, slots)
+        return out
+    return ref_mingru_scan(proj, z_off, x_off, g_off, width, bz, bx, state, cu_q, start_pos, slots, out_dtype)
+
+
+# ---- residual / norms / activation ----------------------------------------------------------------
+
+def dual_norm_add_(x, a, wa, b, wb, eps) -> torch.Tensor:
+    """x += (a / rms(a) * wa + b / rms(b) * wb) / 2, in place on the fp32 residual."""
+    if _gpu(x):
+        native().dual_norm_add(x, a.contiguous(), wa, b.contiguous(), wb, float(eps))
+        return x
+    return ref_dual_norm_add_(x, a, wa, b, wb, eps)
+
+
+def add_norm(x, y, w, eps, out_dtype) -> torch.Tensor:
+    """x += y (in place, fp32; ``y`` may be None), returns x / rms(x) * w."""
+    if _gpu(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        native().add_norm(out, x, y, w, float(eps))
+        return out
+    return ref_add_norm(x, y, w, eps, out_dtype)
+
+
+def limited_glu(gu, limit: float, out_dtype) -> torch.Tensor:
+    """``gu`` [T, 2F] = (gate | up): g = min(gate, limit), u = clamp(up, -limit, limit);
+    returns g * sigmoid(1.702 g) * (u + 1)."""
+    if _gpu(gu):
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=out_dtype, device=gu.device)
+        native().limited_glu(out, gu, float(limit))
+        return out
+    return ref_limited_glu(gu, limit, out_dtype)
+
+
+# ---- the PyTorch statements (CPU tensors; what the kernels are tested against) ---------------------
+
+def _rms(x, eps):
+    return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+
+def ref_shift_norm(x, y, w, eps, mu, state, row_seq, positions, start_pos, slots, out_dtype, shift_state=False):
+    xs = x + y.float() if y is not None else x
+    h = _rms(xs, eps) * w
+    prev = torch.zeros_like(h)
+    prev[1:] = h[:-1]
+    rs = row_seq.long()
+    first = positions == start_pos.long()[rs]
+    prev = torch.where(first[:, None], state[slots.long()[rs]], prev)
+    prev = torch.where((positions == 0)[:, None], torch.zeros_like(prev), prev)
+    out = h + (prev - h) * mu
+    if shift_state:
+        state[slots.long()[rs]] = h
+    return out.to(out_dtype), xs
+
+
+def ref_shift_state_update(x, w, eps, state, cu_q, slots):
+    last = cu_q.long()[1:] - 1
+    state[slots.long()] = _rms(x[last], eps) * w
+
+
+def _rotate_pairs(t, positions, inv_freq):
+    """t [T, n, D] fp32: entry 2i pairs with 2i + 1 on the leading 2 * len(inv_freq) entries."""
+    d = 2 * inv_freq.numel()
+    ang = positions.to(torch.float32)[:, None] * inv_freq[None]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    u, v = t[..., 0:d:2], t[..., 1:d:2]
+    out = t.clone()
+    out[..., 0:d:2] = u * c - v * s
+    out[..., 1:d:2] = v * c + u * s
+    return out
+
+
+def ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping, out_dtype):
+    T = proj.shape[0]
+    H, G, Dk, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    q = proj[:, q_off:q_off + H * Dk].float().reshape(T, H, Dk)
+    k = proj[:, k_off:k_off + G * Dk].float().reshape(T, G, Dk)
+    v = proj[:, k_off:k_off + G * Dk] if spec.value_from_key else proj[:, v_off:v_off + G * Dv]
+    if inv_freq is not None:
+        q, k = _rotate_pairs(q, positions, inv_freq), _rotate_pairs(k, positions, inv_freq)
+    q, k = _rms(q, eps), _rms(k, eps)
+    BS = k_cache.shape[2]
+    blk, off = slot_mapping // BS, slot_mapping % BS
+    k_cache[blk, :, off] = k.to(k_cache.dtype)
+    v_cache[blk, :, off] = v.reshape(T, G, Dv).to(v_cache.dtype)
+    return q.to(out_dtype)
+
+
+def ref_gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale, temp, sink, out_dtype):
+    T, H, Dk = q.shape
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    cq, sp = cu_q.tolist(), start_pos.tolist()
+    hs = torch.full((H,), float(scale), dtype=torch.float32, device=q.device)
+    if temp is not None:
+        hs = hs * temp.float()
+    for s in range(len(sp)):
+        r0, r1 = cq[s], cq[s + 1]
+        if r1 == r0:
+            continue
+        ctx = sp[s] + r1 - r0
+        blocks = block_tables[s, :(ctx + BS - 1) // BS].long()
+        K = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, -1, Dk)[:, :ctx].float()
+        V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, -1, Dv)[:, :ctx].float()
+        qs = q[r0:r1].float().permute(1, 0, 2)                                       # [H, n, Dk]
+        sc = torch.einsum("hnd,hkd->hnk", qs, K.repeat_interleave(H // G, 0)) * hs[:, None, None]
+        qpos = torch.arange(sp[s], ctx, device=q.device)
+        mask = torch.arange(ctx, device=q.device)[None, :] <= qpos[:, None]
+        sc = sc.masked_fill(~mask[None], float("-inf"))
+        m = sc.max(-1, keepdim=True).values
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True) + sink * torch.exp(-m)
+        out[r0:r1] = torch.einsum("hnk,hkd->hnd", e / den, V.repeat_interleave(H // G, 0)).permute(1, 0, 2)
+    return out.reshape(T, H * Dv).to(out_dtype)
+
+
+def ref_mingru_scan(proj, z_off, x_off, g_off, width, bz, bx, state, cu_q, start_pos, slots, out_dtype):
+    z = torch.sigmoid(proj[:, z_off:z_off + width].float() + bz)
+    u = proj[:, x_off:x_off + width].float() + bx
+    c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = torch.nn.functional.silu(proj[:, g_off:g_off + width].float())
+    out = torch.empty(proj.shape[0], width, dtype=torch.float32, device=proj.device)
+    cq, sp, sl = cu_q.tolist(), start_pos.tolist(), slots.tolist()
+    for s in range(len(sp)):
+        if cq[s + 1] == cq[s]:
+            continue
+        S = state[sl[s]].clone() if sp[s] > 0 else torch.zeros(width, dtype=torch.float32, device=proj.device)
+        for r in range(cq[s], cq[s + 1]):
+            S = (1 - z[r]) * S + z[r] * c[r]
+            out[r] = S
+        state[sl[s]] = S
+    return (out * g).to(out_dtype)
+
+
+def ref_dual_norm_add_(x, a, wa, b, wb, eps):
+    x.add_(0.5 * (_rms(a.float(), eps) * wa + _rms(b.float(), eps) * wb))
+    return x
+
+
+def ref_add_norm(x, y, w, eps, out_dtype):
+    if y is not None:
+        x.add_(y.float())
+    return (_rms(x, eps) * w).to(out_dtype)
+
+
+def ref_limited_glu(gu, limit, out_dtype):
+    F = gu.shape[1] // 2
+    g = torch.clamp(gu[:, :F].float(), max=limit)
+    u = torch.clamp(gu[:, F:].float(), -limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1)).to(out_dtype)

@@ -46,9 +46,14 @@ def main(argv=None) -> int:
     from .utils.local_detect import resolve_model
     # the checkpoint's config.json names the model class, as for every engine built on a directory
     model, overrides = resolve_model(a.model, a.model)
-    if device.startswith("cuda") and get_config(model, **overrides).arch == "mupulorn":
-        from .ops import latent
-        latent.ensure_built()          # a fresh checkout compiles this family's kernels here, once
+    if device.startswith("cuda"):      # a fresh checkout compiles the model family's kernels here, once
+        arch = get_config(model, **overrides).arch
+        if arch == "mupulorn":
+            from .ops import latent
+            latent.ensure_built()
+        elif arch == "goganex":
+            from .ops import hybrid
+            hybrid.ensure_built()
     bs = a.block_size
     live = max(1, a.max_live)
     engine = Engine(EngineConfig(model=model, model_overrides=overrides, weights=a.model, dtype=a.dtype, device=device, block_size=bs,
