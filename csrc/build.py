@@ -57,12 +57,26 @@ def latent_ext_path() -> str:
     return os.path.join(PKG, "_C_latent" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
+def hybrid_ext_path() -> str:
+    return os.path.join(PKG, "_C_hybrid" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
 def build_latent(verbose: bool = False, jobs: int = 8) -> str:
     """The latent-attention family's extension ``theroundtaible_amd/_C_latent*.so`` from
     ``csrc/latent/`` — a module of its own, so a checkout that only serves such a model compiles
     three files. Same flags as :func:`build`, plus no packed-fp32 instruction selection."""
-    src_dir = os.path.join(HERE, "latent")
-    bdir = os.path.join(BUILD, "latent")
+    return _build_family("latent", latent_ext_path(), verbose, jobs)
+
+
+def build_hybrid(verbose: bool = False, jobs: int = 8) -> str:
+    """The grouped-attention + recurrence family's extension ``theroundtaible_amd/_C_hybrid*.so``
+    from ``csrc/hybrid/``, a module of its own like :func:`build_latent`'s."""
+    return _build_family("hybrid", hybrid_ext_path(), verbose, jobs)
+
+
+def _build_family(name: str, out: str, verbose: bool = False, jobs: int = 8) -> str:
+    src_dir = os.path.join(HERE, name)
+    bdir = os.path.join(BUILD, name)
     os.makedirs(bdir, exist_ok=True)
     incs, torch_lib, abi = torch_paths()
     py_inc = sysconfig.get_paths()["include"]
@@ -76,17 +90,16 @@ def build_latent(verbose: bool = False, jobs: int = 8) -> str:
         if _newer(src, obj, headers):
             jobs_list.append([HIPCC, "-x", "hip", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
                               "-packed-fp32-ops", *common, "-I", HERE, "-c", src, "-o", obj])
-    bsrc = os.path.join(src_dir, "latent_bindings.cpp")
-    bobj = os.path.join(bdir, "latent_bindings.cpp.o")
+    bsrc = os.path.join(src_dir, f"{name}_bindings.cpp")
+    bobj = os.path.join(bdir, f"{name}_bindings.cpp.o")
     objs.append(bobj)
     if _newer(bsrc, bobj, []):
         jobs_list.append([HIPCC, *common, "-I", py_inc, *sum((["-I", i] for i in incs), []),
-                          "-DTORCH_EXTENSION_NAME=_C_latent", "-DTORCH_API_INCLUDE_EXTENSION_H", "-c", bsrc, "-o", bobj])
+                          f"-DTORCH_EXTENSION_NAME=_C_{name}", "-DTORCH_API_INCLUDE_EXTENSION_H", "-c", bsrc, "-o", bobj])
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         for err in ex.map(_run, jobs_list):
             if verbose and err.strip():
                 print(err)
-    out = latent_ext_path()
     if jobs_list or not os.path.exists(out):
         tmp = out + f".{os.getpid()}.tmp"
         _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp, f"-L{torch_lib}",
@@ -98,6 +111,7 @@ def build_latent(verbose: bool = False, jobs: int = 8) -> str:
 
 def build(verbose: bool = False, jobs: int = 8) -> str:
     build_latent(verbose, jobs)
+    build_hybrid(verbose, jobs)
     os.makedirs(BUILD, exist_ok=True)
     incs, torch_lib, abi = torch_paths()
     py_inc = sysconfig.get_paths()["include"]
@@ -134,6 +148,9 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
 if __name__ == "__main__":
     if "latent" in sys.argv[1:]:
         print(build_latent(verbose="-v" in sys.argv))
+    elif "hybrid" in sys.argv[1:]:
+        print(build_hybrid(verbose="-v" in sys.argv))
     else:
         print(build(verbose="-v" in sys.argv))
         print(latent_ext_path())
+        print(hybrid_ext_path())

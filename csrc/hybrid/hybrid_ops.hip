@@ -1,0 +1,310 @@
+// H1, H2, H4 .. H7: the row-wise kernels of decoders that mix grouped attention with recurrent
+// layers. All math fp32; tensors are bf16 (uint16_t storage) or fp32 as templated. One workgroup
+// per row (H4: per sequence and 256 channels); rows are read twice (the second read hits L1 / L2),
+// never staged in LDS, so any row width runs.
+//
+//   shift_norm        xs = x + y ; h = xs / rms(xs) * w ; out = h + (h_prev - h) * mu
+//                     h_prev: the row above inside a span, the sequence's state at a span's first
+//                     row, zero at position 0; optionally stores h as the new state (decode step)
+//   shift_state       state[slot] = normed last row of every span
+//   qk_prep           rotary pairs (2i, 2i + 1), per-head x / rms(x); keys, values -> paged cache
+//   mingru_scan       z = sigmoid(.), c = u + 1/2 | sigmoid(u); S = (1 - z) S + z c; out = S silu(g)
+//   dual_norm_add     x += (a / rms(a) * wa + b / rms(b) * wb) / 2
+//   add_norm          x += y ; out = x / rms(x) * w
+//   limited_glu       g = min(gate, L), u = clamp(up, -L, L); g * sigmoid(1.702 g) * (u + 1)
+#include "../common.h"
+
+namespace {
+
+using rt::DT;
+
+RT_DEVICE float inv_rms(float ss, int n, float eps) { return 1.0f / sqrtf(ss / (float)n + eps); }
+RT_DEVICE float sigmoidf(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+// block-wide sum of two values at once
+RT_DEVICE void block_sum2(float& a, float& b, float* scratch) {
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  a = rt::wave_sum(a);
+  b = rt::wave_sum(b);
+  __syncthreads();
+  if (lane == 0) {
+    scratch[wid] = a;
+    scratch[16 + wid] = b;
+  }
+  __syncthreads();
+  a = rt::wave_sum(lane < nw ? scratch[lane] : 0.f);
+  b = rt::wave_sum(lane < nw ? scratch[16 + lane] : 0.f);
+}
+
+template <typename OT, typename YT>
+__global__ void __launch_bounds__(1024) shift_norm_kernel(
+    OT* __restrict__ out, float* __restrict__ xs, const float* __restrict__ x, const YT* __restrict__ y,
+    const float* __restrict__ w, const float* __restrict__ mu, float* __restrict__ state,
+    const int* __restrict__ row_seq, const int64_t* __restrict__ positions, const int* __restrict__ start_pos,
+    const int* __restrict__ slots, int W, float eps, int store_state) {
+  __shared__ float scratch[32];
+  const int t = blockIdx.x;
+  const int s = row_seq[t];
+  const int64_t pos = positions[t];
+  const bool first = pos == (int64_t)start_pos[s];      // first row of its span in this launch
+  const float* xr = x + (size_t)t * W;
+  const YT* yr = y ? y + (size_t)t * W : nullptr;
+  const float* xp = xr - W;                              // only read when !first (then t > 0)
+  const YT* yp = yr ? yr - W : nullptr;
+  float* st = state + (size_t)slots[s] * W;
+  float ss = 0.f, sp = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+    ss += v * v;
+    if (!first) {
+      const float u = xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f);
+      sp += u * u;
+    }
+  }
+  block_sum2(ss, sp, scratch);
+  const float kc = inv_rms(ss, W, eps), kp = inv_rms(sp, W, eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+    const float h = v * kc * w[c];
+    float hp;
+    if (!first) hp = (xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f)) * kp * w[c];
+    else hp = pos > 0 ? st[c] : 0.f;
+    DT<OT>::store(out + (size_t)t * W + c, h + (hp - h) * mu[c]);
+    if (yr) xs[(size_t)t * W + c] = v;
+    if (store_state) st[c] = h;
+  }
+}
+
+__global__ void __launch_bounds__(1024) shift_state_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                           float* __restrict__ state, const int* __restrict__ cu_q,
+                                                           const int* __restrict__ slots, int W, float eps) {
+  __shared__ float scratch[16];
+  const int s = blockIdx.x;
+  const int n = cu_q[s + 1] - cu_q[s];
+  if (n <= 0) return;
+  const float* xr = x + (size_t)(cu_q[s + 1] - 1) * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) ss += xr[c] * xr[c];
+  const float k = inv_rms(rt::block_sum(ss, scratch), W, eps);
+  float* st = state + (size_t)slots[s] * W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) st[c] = xr[c] * k * w[c];
+}
+
+// One wave per head unit: units 0 .. H - 1 are query heads, H .. H + G - 1 key heads (each also
+// writes its value head). A lane holds entries lane, lane + 64, ... of the head (at most 4).
+template <typename T>
+__global__ void __launch_bounds__(256) qk_prep_kernel(
+    T* __restrict__ q, const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int v_from_k,
+    const float* __restrict__ inv_freq, int rot_dims, float eps, const int64_t* __restrict__ positions,
+    T* __restrict__ kc, T* __restrict__ vc, const int64_t* __restrict__ slot_mapping, int H, int G, int Dk, int Dv,
+    int BS) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const float pos = (float)positions[t];
+  const int64_t slot = slot_mapping[t];
+  const int64_t blk = slot / BS;
+  const int off = (int)(slot - blk * BS);
+  const T* row = proj + (size_t)t * stride;
+  for (int u = wave; u < H + G; u += nw) {
+    const bool is_q = u < H;
+    const T* src = row + (is_q ? q_off + u * Dk : k_off + (u - H) * Dk);
+    float val[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = lane + 64 * j;
+      float r = 0.f;
+      if (d < Dk) {
+        const float a = DT<T>::load(src + d);
+        r = a;
+        if (d < rot_dims) {
+          const float b = DT<T>::load(src + (d ^ 1));
+          float sn, cs;
+          sincosf(pos * inv_freq[d >> 1], &sn, &cs);
+          r = (d & 1) ? a * cs + b * sn : a * cs - b * sn;
+        }
+      }
+      val[j] = r;
+      ss += r * r;
+    }
+    const float k = inv_rms(rt::wave_sum(ss), Dk, eps);
+    T* dst = is_q ? q + ((size_t)t * H + u) * Dk : kc + (((size_t)blk * G + (u - H)) * BS + off) * Dk;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = lane + 64 * j;
+      if (d < Dk) DT<T>::store(dst + d, val[j] * k);
+    }
+    if (!is_q) {
+      const int g = u - H;
+      const T* vs = v_from_k ? src : row + v_off + g * Dv;
+      T* vd = vc + (((size_t)blk * G + g) * BS + off) * Dv;
+      for (int d = lane; d < Dv; d += 64) vd[d] = vs[d];
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) mingru_scan_kernel(
+    T* __restrict__ out, const T* __restrict__ proj, int stride, int z_off, int x_off, int g_off, int width,
+    const float* __restrict__ bz, const float* __restrict__ bx, float* __restrict__ state,
+    const int* __restrict__ cu_q, const int* __restrict__ start_pos, const int* __restrict__ slots) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int r0 = cu_q[s], r1 = cu_q[s + 1];
+  if (c >= width || r1 <= r0) return;
+  float* st = state + (size_t)slots[s] * width + c;
+  float S = start_pos[s] > 0 ? *st : 0.f;
+  const float bzc = bz[c], bxc = bx[c];
+  for (int r = r0; r < r1; ++r) {
+    const T* row = proj + (size_t)r * stride;
+    const float z = sigmoidf(DT<T>::load(row + z_off + c) + bzc);
+    const float u = DT<T>::load(row + x_off + c) + bxc;
+    const float cand = u >= 0.f ? u + 0.5f : sigmoidf(u);
+    const float g = DT<T>::load(row + g_off + c);
+    S = (1.0f - z) * S + z * cand;
+    DT<T>::store(out + (size_t)r * width + c, S * (g * sigmoidf(g)));
+  }
+  *st = S;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(1024) dual_norm_add_kernel(float* __restrict__ x, const T* __restrict__ a,
+                                                             const float* __restrict__ wa, const T* __restrict__ b,
+                                                             const float* __restrict__ wb, int W, float eps) {
+  __shared__ float scratch[32];
+  const T* ar = a + (size_t)blockIdx.x * W;
+  const T* br = b + (size_t)blockIdx.x * W;
+  float sa = 0.f, sb = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float u = DT<T>::load(ar + c), v = DT<T>::load(br + c);
+    sa += u * u;
+    sb += v * v;
+  }
+  block_sum2(sa, sb, scratch);
+  const float ka = inv_rms(sa, W, eps), kb = inv_rms(sb, W, eps);
+  float* xr = x + (size_t)blockIdx.x * W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    xr[c] += 0.5f * (DT<T>::load(ar + c) * ka * wa[c] + DT<T>::load(br + c) * kb * wb[c]);
+}
+
+template <typename OT, typename YT>
+__global__ void __launch_bounds__(1024) add_norm_kernel(OT* __restrict__ out, float* __restrict__ x,
+                                                        const YT* __restrict__ y, const float* __restrict__ w, int W,
+                                                        float eps) {
+  __shared__ float scratch[16];
+  float* xr = x + (size_t)blockIdx.x * W;
+  const YT* yr = y ? y + (size_t)blockIdx.x * W : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+    ss += v * v;
+  }
+  const float k = inv_rms(rt::block_sum(ss, scratch), W, eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+    if (yr) xr[c] = v;
+    DT<OT>::store(out + (size_t)blockIdx.x * W + c, v * k * w[c]);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) limited_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t rows,
+                                                          int F, float limit) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * F) return;
+  const int64_t r = i / F;
+  const int c = (int)(i - r * F);
+  const float g = fminf(DT<T>::load(gu + r * 2 * F + c), limit);
+  const float u = fminf(fmaxf(DT<T>::load(gu + r * 2 * F + F + c), -limit), limit);
+  DT<T>::store(out + i, g * sigmoidf(1.702f * g) * (u + 1.0f));
+}
+
+int row_threads(int W) {
+  int t = 64;
+  while (t < 1024 && t * 4 < W) t *= 2;
+  return t;
+}
+
+}  // namespace
+
+void launch_shift_norm(void* out, float* xs, const float* x, const void* y, const float* w, const float* mu,
+                       float* state, const int* row_seq, const int64_t* positions, const int* start_pos,
+                       const int* slots, int T, int W, float eps, bool out_bf, bool y_bf, bool store_state,
+                       hipStream_t stream) {
+  if (T <= 0) return;
+  const int th = row_threads(W);
+#define RT_SN(OT, YT)                                                                                              \
+  shift_norm_kernel<OT, YT><<<T, th, 0, stream>>>((OT*)out, xs, x, (const YT*)y, w, mu, state, row_seq, positions, \
+                                                  start_pos, slots, W, eps, store_state ? 1 : 0)
+  if (out_bf) {
+    if (y_bf) RT_SN(uint16_t, uint16_t); else RT_SN(uint16_t, float);
+  } else {
+    if (y_bf) RT_SN(float, uint16_t); else RT_SN(float, float);
+  }
+#undef RT_SN
+}
+
+void launch_shift_state(const float* x, const float* w, float* state, const int* cu_q, const int* slots, int S, int W,
+                        float eps, hipStream_t stream) {
+  if (S <= 0) return;
+  shift_state_kernel<<<S, row_threads(W), 0, stream>>>(x, w, state, cu_q, slots, W, eps);
+}
+
+void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off, int v_off, bool v_from_k,
+                    const float* inv_freq, int rot_dims, float eps, const int64_t* positions, void* kc, void* vc,
+                    const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf,
+                    hipStream_t stream) {
+  if (T <= 0) return;
+  if (bf)
+    qk_prep_kernel<uint16_t><<<T, 256, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
+                                                    v_from_k, inv_freq, rot_dims, eps, positions, (uint16_t*)kc,
+                                                    (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS);
+  else
+    qk_prep_kernel<float><<<T, 256, 0, stream>>>((float*)q, (const float*)proj, stride, q_off, k_off, v_off, v_from_k,
+                                                 inv_freq, rot_dims, eps, positions, (float*)kc, (float*)vc,
+                                                 slot_mapping, H, G, Dk, Dv, BS);
+}
+
+void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
+                        const float* bz, const float* bx, float* state, const int* cu_q, const int* start_pos,
+                        const int* slots, int S, bool bf, hipStream_t stream) {
+  if (S <= 0 || width <= 0) return;
+  const int th = width >= 256 ? 256 : 64;
+  dim3 grid(S, (width + th - 1) / th);
+  if (bf)
+    mingru_scan_kernel<uint16_t><<<grid, th, 0, stream>>>((uint16_t*)out, (const uint16_t*)proj, stride, z_off, x_off,
+                                                          g_off, width, bz, bx, state, cu_q, start_pos, slots);
+  else
+    mingru_scan_kernel<float><<<grid, th, 0, stream>>>((float*)out, (const float*)proj, stride, z_off, x_off, g_off,
+                                                       width, bz, bx, state, cu_q, start_pos, slots);
+}
+
+void launch_dual_norm_add(float* x, const void* a, const float* wa, const void* b, const float* wb, int T, int W,
+                          float eps, bool bf, hipStream_t stream) {
+  if (T <= 0) return;
+  if (bf)
+    dual_norm_add_kernel<uint16_t><<<T, row_threads(W), 0, stream>>>(x, (const uint16_t*)a, wa, (const uint16_t*)b, wb,
+                                                                     W, eps);
+  else
+    dual_norm_add_kernel<float><<<T, row_threads(W), 0, stream>>>(x, (const float*)a, wa, (const float*)b, wb, W, eps);
+}
+
+void launch_add_norm(void* out, float* x, const void* y, const float* w, int T, int W, float eps, bool out_bf,
+                     bool y_bf, hipStream_t stream) {
+  if (T <= 0) return;
+  const int th = row_threads(W);
+#define RT_AN(OT, YT) add_norm_kernel<OT, YT><<<T, th, 0, stream>>>((OT*)out, x, (const YT*)y, w, W, eps)
+  if (out_bf) {
+    if (y_bf) RT_AN(uint16_t, uint16_t); else RT_AN(uint16_t, float);
+  } else {
+    if (y_bf) RT_AN(float, uint16_t); else RT_AN(float, float);
+  }
+#undef RT_AN
+}
+
+void launch_limited_glu(void* out, const void* gu, int64_t rows, int F, float limit, bool bf, hipStream_t stream) {
+  const int64_t n = rows * F;
+  if (n <= 0) return;
+  const int blocks = (int)((n + 255) / 256);
+  if (bf) limited_glu_kernel<uint16_t><<<blocks, 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)gu, rows, F, limit);
+  else limited_glu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, rows, F, limit);
+}
