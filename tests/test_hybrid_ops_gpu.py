@@ -1,0 +1,157 @@
+"""Every HIP kernel of ``csrc/hybrid/`` against its PyTorch statement (``ops/hybrid.py`` ``ref_*``,
+run on fp32 CPU copies of the same inputs), at sizes that are not multiples of the kernels' tile
+shapes, in fp32 and bf16."""
+import pytest
+import torch
+
+from theroundtaible_amd.models.config import GroupedAttentionSpec
+from theroundtaible_amd.ops import hybrid as Hy
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dt):
+    return dict(rtol=2e-2, atol=2e-2) if dt == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
+
+
+def spans(lens, starts):
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    row_seq = torch.repeat_interleave(torch.arange(len(lens), dtype=torch.int32), torch.tensor(lens))
+    pos = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)])
+    return cu, row_seq, pos, torch.tensor(starts, dtype=torch.int32)
+
+
+def gpu(*ts):
+    return [t.to(DEV) if t is not None else None for t in ts]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("W", [20, 192, 1100])
+def test_shift_norm_and_state(dt, W):
+    Hy.native()
+    g = torch.Generator().manual_seed(W)
+    lens, starts = [5, 1, 1, 9], [0, 0, 7, 3]
+    cu, row_seq, pos, sp = spans(lens, starts)
+    T = sum(lens)
+    slots = torch.tensor([2, 0, 3, 1], dtype=torch.int32)
+    x, y = torch.randn(T, W, generator=g), torch.randn(T, W, generator=g).to(dt)
+    w, mu, state = torch.rand(W, generator=g) + 0.5, torch.rand(W, generator=g), torch.randn(5, W, generator=g)
+    for yy in (y, None):
+        st_c, st_g = state.clone(), state.clone().to(DEV)
+        want, xs = Hy.ref_shift_norm(x.clone(), yy, w, 1e-5, mu, st_c, row_seq, pos, sp, slots, torch.float32)
+        Hy.ref_shift_state_update(xs, w, 1e-5, st_c, cu, slots)
+        got, xg = Hy.shift_norm(*gpu(x, yy, w), 1e-5, *gpu(mu, st_g, row_seq, pos, sp, slots), dt)
+        Hy.shift_state_update(xg, w.to(DEV), 1e-5, st_g, cu.to(DEV), slots.to(DEV))
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+        torch.testing.assert_close(xg.cpu(), xs, rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-5, atol=1e-5)
+    # one row per sequence, the state stored by the same launch
+    B = 4
+    cu, row_seq, pos, sp = spans([1] * B, [0, 4, 9, 1])
+    st_c, st_g = state.clone(), state.clone().to(DEV)
+    want, _ = Hy.ref_shift_norm(x[:B].clone(), None, w, 1e-5, mu, st_c, row_seq, pos, sp, slots, torch.float32, True)
+    got, _ = Hy.shift_norm(*gpu(x[:B], None, w), 1e-5, *gpu(mu, st_g, row_seq, pos, sp, slots), dt, shift_state=True)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+    torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 2, 12, 20, 6, False), (3, 3, 72, 72, 0, True), (5, 1, 130, 200, 130, False),
+                                   (2, 1, 1, 1, 0, False)])
+def test_qk_prep(dt, shape):
+    H, G, Dk, Dv, rot, vk = shape
+    g = torch.Generator().manual_seed(Dk)
+    T, BS, nb = 11, 4, 6
+    spec = GroupedAttentionSpec(H, G, Dk, Dv, 1.0, value_from_key=vk)
+    N = 3 + H * Dk + G * Dk + (0 if vk else G * Dv)
+    proj = torch.randn(T, N, generator=g).to(dt)
+    inv = (torch.rand(rot // 2, generator=g) if rot else None)
+    pos = torch.tensor([0, 1, 2, 3, 40, 41, 900, 901, 5000, 70000, 7])
+    slots = torch.randperm(nb * BS, generator=g)[:T]
+    kc, vc = torch.zeros(nb, G, BS, Dk, dtype=dt), torch.zeros(nb, G, BS, Dv, dtype=dt)
+    want = Hy.ref_qk_prep(proj, spec, 3, 3 + H * Dk, 3 + (H + G) * Dk, inv, 1e-5, pos, kc, vc, slots, torch.float32)
+    kg, vg = torch.zeros_like(kc).to(DEV), torch.zeros_like(vc).to(DEV)
+    got = Hy.qk_prep(proj.to(DEV), spec, 3, 3 + H * Dk, 3 + (H + G) * Dk, inv.to(DEV) if rot else None, 1e-5, pos.to(DEV),
+                     kg, vg, slots.to(DEV), dt)
+    # (angles of far positions in fp32: the two sides round p * f alike, the sine differs by ulps)
+    t = dict(rtol=2e-2, atol=2e-2) if dt == torch.bfloat16 else dict(rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(got.float().cpu(), want, **t)
+    torch.testing.assert_close(kg.float().cpu(), kc.float(), **t)
+    torch.testing.assert_close(vg.float().cpu(), vc.float(), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("shape", [(6, 2, 12, 12, 16), (4, 4, 48, 20, 64), (5, 1, 72, 132, 8), (40, 1, 8, 8, 16),
+                                   (8, 2, 128, 128, 32), (2, 1, 256, 256, 16)])
+def test_gqa_attention_varlen_and_split(dt, shape):
+    H, G, Dk, Dv, BS = shape
+    g = torch.Generator().manual_seed(H * Dk)
+    lens, starts = [37, 1, 2, 70], [0, 130, 63, 5]
+    cu, _, _, sp = spans(lens, starts)
+    T = sum(lens)
+    ctx = [s + n for s, n in zip(starts, lens)]
+    nblk = [(c + BS - 1) // BS for c in ctx]
+    nb = sum(nblk) + 2
+    perm = torch.randperm(nb, generator=g).tolist()
+    bt = torch.zeros(len(lens), max(nblk), dtype=torch.int32)
+    for s, n in enumerate(nblk):
+        bt[s, :n] = torch.tensor([perm.pop() for _ in range(n)])
+    kc = (torch.randn(nb, G, BS, Dk, generator=g) * 0.5).to(dt)
+    vc = torch.randn(nb, G, BS, Dv, generator=g).to(dt)
+    q = torch.randn(T, H, Dk, generator=g).to(dt)
+    temp = torch.rand(H, generator=g) + 0.5
+    for sink, tp in ((1.0, temp), (0.0, None)):
+        want = Hy.ref_gqa_attention(q.float(), kc.float(), vc.float(), bt, cu, sp, 0.3, tp, sink, torch.float32)
+        got = Hy.gqa_attention(*gpu(q, kc, vc, bt, cu, sp), 0.3, tp.to(DEV) if tp is not None else None, sink)
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+    # one row per sequence with split keys (2, 7, 32 ranges)
+    B = len(lens)
+    last = torch.tensor([c - 1 for c in ctx], dtype=torch.int32)
+    rows = torch.tensor([int(cu[s + 1]) - 1 for s in range(B)])
+    cu1 = torch.arange(B + 1, dtype=torch.int32)
+    want = Hy.ref_gqa_attention(q[rows].float(), kc.float(), vc.float(), bt, cu1, last, 0.3, temp, 1.0, torch.float32)
+    tiles = torch.stack([torch.arange(B), torch.arange(B)], 1).to(torch.int32)
+    for splits in (2, 7, 32):
+        got = Hy.gqa_attention(*gpu(q[rows].contiguous(), kc, vc, bt, cu1, last), 0.3, temp.to(DEV), 1.0, tiles=tiles.to(DEV),
+                               num_splits=splits)
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("width", [7, 224, 300])
+def test_mingru_scan(dt, width):
+    g = torch.Generator().manual_seed(width)
+    lens, starts = [33, 1, 1, 130], [0, 0, 12, 3]
+    cu, _, _, sp = spans(lens, starts)
+    T = sum(lens)
+    slots = torch.tensor([1, 3, 0, 2], dtype=torch.int32)
+    proj = torch.randn(T, 5 + 3 * width, generator=g).to(dt)
+    bz, bx, state = torch.randn(width, generator=g), torch.randn(width, generator=g), torch.randn(4, width, generator=g)
+    st_c, st_g = state.clone(), state.clone().to(DEV)
+    want = Hy.ref_mingru_scan(proj, 5, 5 + 2 * width, 5 + width, width, bz, bx, st_c, cu, sp, slots, torch.float32)
+    got = Hy.mingru_scan(proj.to(DEV), 5, 5 + 2 * width, 5 + width, width, *gpu(bz, bx, st_g, cu, sp, slots), dt)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+    torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_normed_adds_and_activation(dt):
+    g = torch.Generator().manual_seed(0)
+    T, W, F = 13, 200, 77
+    x = torch.randn(T, W, generator=g)
+    a, b = torch.randn(T, W, generator=g).to(dt), (3 * torch.randn(T, W, generator=g)).to(dt)
+    wa, wb = torch.rand(W, generator=g), torch.rand(W, generator=g)
+    xg = x.clone().to(DEV)
+    Hy.dual_norm_add_(xg, *gpu(a, wa, b, wb), 1e-5)
+    torch.testing.assert_close(xg.cpu(), Hy.ref_dual_norm_add_(x.clone(), a, wa, b, wb, 1e-5), rtol=1e-5, atol=1e-5)
+    for y in (a, None):
+        xc, xg = x.clone(), x.clone().to(DEV)
+        want = Hy.ref_add_norm(xc, y, wa, 1e-5, torch.float32)
+        got = Hy.add_norm(xg, y.to(DEV) if y is not None else None, wa.to(DEV), 1e-5, dt)
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+        torch.testing.assert_close(xg.cpu(), xc, rtol=1e-6, atol=1e-6)
+    gu = (2 * torch.randn(T, 2 * F, generator=g)).to(dt)
+    torch.testing.assert_close(Hy.limited_glu(gu.to(DEV), 1.5, dt).float().cpu(), Hy.ref_limited_glu(gu, 1.5, torch.float32),
+                               **tol(dt))
