@@ -114,7 +114,7 @@ def parse():
                         "JSON (parallel/costmodel.py default_calibration, $ROUNDTABLE_CALIBRATION)")
     p.add_argument("--arch-compare", default="",
                    help="instead of the headline workload: prefill and decode throughput of model pairs "
-                        "'a:b,c:d' (e.g. mupulorn-8b:llama3-8b,mupulorn-1b:llama3.2-1b), each model with "
+                        "'a:b,c:d' (e.g. mupulorn-8b:llama3-8b,goganex-8b:llama3-8b,goganex-1b:llama3.2-1b), each model with "
                         "--compare-layers layers and random weights, through the same engine entry points; "
                         "prints one JSON line per model")
     p.add_argument("--compare-layers", type=int, default=4)

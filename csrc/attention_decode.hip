@@ -186,6 +186,7 @@ __global__ void __launch_bounds__(1024) decode_combine_kernel(AttnArgs p) {
 #pragma unroll
     for (int x = 8; x < 64; x <<= 1) xmerge(x, w & (x >> 3));
     if (w == 0) {
+      if (p.sink > 0.f) L += p.sink * exp2f(-M);
       const float inv = L > 0.f ? 1.f / L : 0.f;
       store_bf16x4(p.out + (size_t)row * D + d0, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv, false);
     }
@@ -202,7 +203,8 @@ __global__ void __launch_bounds__(1024) decode_combine_kernel(AttnArgs p) {
 int launch_paged_decode(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                         const int* ctx_lens, float* part_o, float* part_ml, int* counters, int B, int Hq, int Hkv,
                         int D, int max_blocks, float scale, int num_splits, const int* groups, int slot_stride,
-                        hipStream_t stream, int defer_combine, int* deferred, const int* plan, int plan_stride) {
+                        hipStream_t stream, int defer_combine, int* deferred, const int* plan, int plan_stride,
+                        float sink) {
   if (deferred != nullptr) *deferred = 0;
   if (B == 0) return 0;
   if (Hq % Hkv || Hq / Hkv > 16) return -1;
@@ -216,6 +218,7 @@ int launch_paged_decode(void* out, const void* q, const void* k_cache, const voi
                       groups, groups != nullptr ? slot_stride : 0};
   static const int probe = getenv("RT_ATTN_PROBE") ? atoi(getenv("RT_ATTN_PROBE")) : 0;
   args.probe = probe;
+  args.sink = sink;
   if (plan != nullptr) {
     if (plan_stride <= PLAN_HDR) return -5;
     args.plan = plan;

@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(256) prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int Hq, int Hkv, int max_blocks,
-    float scale_log2, int rows_per_tile) {
+    float scale_log2, int rows_per_tile, float sink) {
   using C = PrefillCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -218,7 +218,9 @@ __global__ void __launch_bounds__(256) prefill_kernel(
     l += __shfl_xor(l, 32, 64);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float li = __shfl(l, 4 * g + i, 64);
+      float li = __shfl(l, 4 * g + i, 64);
+      const float mi = __shfl(m[hh], 4 * g + i, 64);
+      if (sink > 0.f) li += sink * exp2f(-mi);     // a key of score 0 without a value
       const int row = wrow0 + 4 * g + i;
       if (row < q_end && row < row0 + rows_per_tile && head0 + hh < hk * G + G) {
         uint16_t* orow = out + ((size_t)row * Hq + head0 + hh) * D;
@@ -235,7 +237,7 @@ int prefill32_rows(int G);
 int launch_prefill32(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                      const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv,
                      int max_blocks, float scale, hipStream_t stream, int map_stride, const int* cmap, int n_split,
-                     float* part_o, float* part_ml);
+                     float* part_o, float* part_ml, float sink);
 
 // D = 128 with G <= 8 (a non-power-of-two group in the next power of two of head slots) runs the
 // 32x32-MFMA kernel (attention_prefill32.hip) unless
@@ -254,20 +256,20 @@ int prefill_rows_per_tile(int G, int D) {
 // q [T, Hq, D]; tile_map [n_tiles, 2] int32 (sequence, first row).
 int launch_prefill(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                    const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv, int D,
-                   int max_blocks, float scale, hipStream_t stream) {
+                   int max_blocks, float scale, hipStream_t stream, float sink) {
   if (n_tiles == 0) return 0;
   const int G = Hq / Hkv;
   if (Hq % Hkv || G < 1 || G > 16) return -1;
   if (use_prefill32(G, D))
     return launch_prefill32(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, n_tiles, Hq, Hkv,
-                            max_blocks, scale, stream, 2, nullptr, 0, nullptr, nullptr);
+                            max_blocks, scale, stream, 2, nullptr, 0, nullptr, nullptr, sink);
   const int rows = prefill_rows_per_tile(G, D);
   dim3 grid(n_tiles, Hkv), block(256);
   const float sl2 = scale * LOG2E;
 #define RT_PF(DD, HH)                                                                                            \
   hipLaunchKernelGGL((prefill_kernel<DD, HH>), grid, block, 2 * PrefillCfg<DD>::STAGE, stream, (uint16_t*)out,   \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
-                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows)
+                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, sink)
   const int hpw = G > 4 ? (G + 3) / 4 : 1;
   if (D == 128) {
     if (hpw == 1) RT_PF(128, 1);
@@ -298,7 +300,7 @@ int launch_prefill_split(void* out, const void* q, const void* k_cache, const vo
   const int G = Hq / Hkv;
   if (Hq % Hkv || !use_prefill32(G, D)) return -1;
   return launch_prefill32(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, items, n_items, Hq, Hkv,
-                          max_blocks, scale, stream, 5, cmap, n_split, part_o, part_ml);
+                          max_blocks, scale, stream, 5, cmap, n_split, part_o, part_ml, 0.f);
 }
 
 int prefill_split_supported(int G, int D) { return use_prefill32(G, D) ? 1 : 0; }

@@ -110,7 +110,8 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int Hq, int Hkv, int max_blocks,
-    float scale_log2, int rows_per_tile, int map_stride, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float scale_log2, int rows_per_tile, int map_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
+    float sink) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];   // 68 KiB: static (> 64 KiB)
   // XCD-aware order: workgroups are dealt round-robin over the 8 XCDs (id mod 8), so with
   // id = tile * Hkv + hk every workgroup of kv head hk lands on XCD hk (Hkv = 8): that head's
@@ -337,6 +338,7 @@ __global__ void __launch_bounds__(NW * 64) prefill32_kernel(
     return;
   }
   if (head_ok && row < q_end && row < row0 + rows_per_tile) {
+    if (sink > 0.f) lsum += sink * exp2f(-m);     // a key of score 0 without a value (whole tiles only)
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
     uint16_t* orow = out + ((size_t)row * Hq + head) * D;
 #pragma unroll
@@ -427,12 +429,13 @@ int prefill32_rows(int G) {
 int launch_prefill32(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                      const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv,
                      int max_blocks, float scale, hipStream_t stream, int map_stride, const int* cmap, int n_split,
-                     float* part_o, float* part_ml) {
+                     float* part_o, float* part_ml, float sink) {
   const int G = Hq / Hkv;
   const int rows = prefill32_rows(G);
   if (rows == 0) return -1;
   if (map_stride != 2 && map_stride != 5) return -2;
   if (map_stride == 5 && n_split > 0 && (cmap == nullptr || part_o == nullptr || part_ml == nullptr)) return -3;
+  if (map_stride == 5 && sink != 0.f) return -4;    // the key-split combine has no sink term
   const float sl2 = scale * LOG2E;
   dim3 grid(n_tiles * Hkv);
   static const int depth = [] {
@@ -442,10 +445,10 @@ int launch_prefill32(void* out, const void* q, const void* k_cache, const void* 
 #define RT_P32(GG, NWV)                                                                                          \
   if (depth == 1) hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 1>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out, \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
-                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml);          \
+                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml, sink);          \
   else hipLaunchKernelGGL((prefill32_kernel<GG, NWV, 2>), grid, dim3(64 * NWV), 0, stream, (uint16_t*)out,              \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, cu_q, \
-                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml);          \
+                     start_pos, tile_map, Hq, Hkv, max_blocks, sl2, rows, map_stride, part_o, part_ml, sink);          \
   if (map_stride == 5 && n_split > 0)                                                                            \
     hipLaunchKernelGGL((prefill32_combine_kernel<GG, NWV>), dim3(n_split * Hkv, D / 16), dim3(32 * NWV), 0, stream, \
                        (uint16_t*)out, cmap, cu_q, (const float*)part_o, (const float*)part_ml, Hq, Hkv, rows)

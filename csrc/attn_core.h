@@ -132,6 +132,9 @@ struct AttnArgs {
   // (sequence, split), PLAN_HDR header ints then the item's block ids, plan_stride ints per item
   const int* plan = nullptr;
   int plan_stride = 0;
+  // softmax sink: a constant added to every row's denominator as sink * exp(0 - max) (a key of
+  // score 0 without a value); 0 = ordinary softmax. Added once, where a row is normalised.
+  float sink = 0.f;
 };
 
 // The key range of work item (sequence b, split) — shared chunk of its group's prefix, then its
@@ -496,6 +499,7 @@ RT_DEVICE bool attn_item(const AttnArgs& P, int bh, int split, AttnSmem<D, GM, W
       }
     }
     if (nslots == 1) {
+      if (P.sink > 0.f) L += P.sink * exp2f(-M);
       const float inv = L > 0.f ? 1.f / L : 0.f;
       store_bf16x4(out + (q0 + row) * D + d0, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv, SC1);
     } else {
@@ -630,6 +634,7 @@ RT_DEVICE bool attn_item(const AttnArgs& P, int bh, int split, AttnSmem<D, GM, W
     }
   }
   if (grp == 0) {
+    if (P.sink > 0.f) Lr += P.sink * exp2f(-Mr);
     const float inv = Lr > 0.f ? 1.f / Lr : 0.f;
     store_bf16x4(out + (q0 + row) * D + d0, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv, SC1);
   }

@@ -18,7 +18,8 @@ void launch_gelu(void* out, const void* x, int64_t n, hipStream_t stream);
 int launch_paged_decode(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                         const int* ctx_lens, float* part_o, float* part_ml, int* counters, int B, int Hq, int Hkv,
                         int D, int max_blocks, float scale, int num_splits, const int* groups, int slot_stride,
-                        hipStream_t stream, int defer_combine, int* deferred, const int* plan, int plan_stride);
+                        hipStream_t stream, int defer_combine, int* deferred, const int* plan, int plan_stride,
+                        float sink);
 int launch_attn_plan(int* plan, int plan_stride, const int* block_tables, const int* ctx_lens, const int* groups,
                      int B, int Hq, int Hkv, int max_blocks, int num_splits, hipStream_t stream);
 int prefill_rows_per_tile(int G, int D);
@@ -29,7 +30,7 @@ int launch_prefill_split(void* out, const void* q, const void* k_cache, const vo
 int prefill_split_supported(int G, int D);
 int launch_prefill(void* out, const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                    const int* cu_q, const int* start_pos, const int* tile_map, int n_tiles, int Hq, int Hkv, int D,
-                   int max_blocks, float scale, hipStream_t stream);
+                   int max_blocks, float scale, hipStream_t stream, float sink);
 int launch_sample(int64_t* out, const void* logits, bool is_bf16, int B, int V, int64_t ld_row,
                   const float* temperature, const float* top_p, const int* top_k, const int64_t* seeds,
                   const int64_t* offsets, float* ws, hipStream_t stream, const void* advance);
@@ -172,7 +173,7 @@ int64_t paged_attention_decode(torch::Tensor out, torch::Tensor q, torch::Tensor
                                torch::Tensor block_tables, torch::Tensor ctx_lens, double scale, int64_t num_splits,
                                torch::Tensor part_o, torch::Tensor part_ml, torch::Tensor counters,
                                c10::optional<torch::Tensor> groups, int64_t slot_stride, bool defer_combine,
-                               c10::optional<torch::Tensor> plan, int64_t plan_stride) {
+                               c10::optional<torch::Tensor> plan, int64_t plan_stride, double sink) {
   check_bf16(out, "out");
   check_bf16(q, "q");
   TORCH_CHECK(q.dim() == 3, "q must be [B, Hq, D]");
@@ -209,7 +210,7 @@ int64_t paged_attention_decode(torch::Tensor out, torch::Tensor q, torch::Tensor
                                      part_ml.data_ptr<float>(), counters.data_ptr<int>(), (int)B, (int)Hq,
                                      (int)k_cache.size(1), (int)D,
                                      (int)block_tables.size(1), (float)scale, (int)num_splits, gp, (int)stride,
-                                     cur_stream(), defer_combine ? 1 : 0, &deferred, pp, (int)plan_stride);
+                                     cur_stream(), defer_combine ? 1 : 0, &deferred, pp, (int)plan_stride, (float)sink);
   TORCH_CHECK(rc == 0, "paged_attention_decode: unsupported configuration (rc=", rc, ")");
   return deferred;
 }
@@ -236,7 +237,7 @@ void attn_plan(torch::Tensor plan, int64_t plan_stride, torch::Tensor block_tabl
 
 void prefill_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
                        torch::Tensor block_tables, torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor tile_map,
-                       double scale) {
+                       double scale, double sink) {
   check_bf16(out, "out");
   check_bf16(q, "q");
   TORCH_CHECK(q.dim() == 3, "q must be [T, Hq, D]");
@@ -252,7 +253,7 @@ void prefill_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
   const int rc = launch_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), cu_q.data_ptr<int>(), start_pos.data_ptr<int>(),
                                 tile_map.data_ptr<int>(), (int)tile_map.size(0), (int)Hq, (int)k_cache.size(1), (int)D,
-                                (int)block_tables.size(1), (float)scale, cur_stream());
+                                (int)block_tables.size(1), (float)scale, cur_stream(), (float)sink);
   TORCH_CHECK(rc == 0, "prefill_attention: unsupported configuration (rc=", rc, ")");
 }
 
@@ -729,11 +730,13 @@ PYBIND11_MODULE(_C, m) {
         py::arg("v_cache"), py::arg("block_tables"), py::arg("ctx_lens"), py::arg("scale"), py::arg("num_splits"),
         py::arg("part_o"), py::arg("part_ml"), py::arg("counters"), py::arg("groups") = py::none(),
         py::arg("slot_stride") = 0, py::arg("defer_combine") = false, py::arg("plan") = py::none(),
-        py::arg("plan_stride") = 0);
+        py::arg("plan_stride") = 0, py::arg("sink") = 0.0);
   m.def("attn_plan", &attn_plan, py::arg("plan"), py::arg("plan_stride"), py::arg("block_tables"),
         py::arg("ctx_lens"), py::arg("groups"), py::arg("B"), py::arg("Hq"), py::arg("Hkv"), py::arg("num_splits"));
   m.def("prefill_rows_per_tile", &prefill_rows_per_tile, py::arg("G"), py::arg("D") = 128);
-  m.def("prefill_attention", &prefill_attention);
+  m.def("prefill_attention", &prefill_attention, py::arg("out"), py::arg("q"), py::arg("k_cache"), py::arg("v_cache"),
+        py::arg("block_tables"), py::arg("cu_q"), py::arg("start_pos"), py::arg("tile_map"), py::arg("scale"),
+        py::arg("sink") = 0.0);
   m.def("prefill_attention_split", &prefill_attention_split);
   m.def("prefill_split_supported", &prefill_split_supported, py::arg("G"), py::arg("D") = 128);
   m.def("silu_and_mul", &silu_and_mul);

@@ -14,8 +14,8 @@ void launch_shift_state(const float* x, const float* w, float* state, const int*
                         float eps, hipStream_t stream);
 void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off, int v_off, bool v_from_k,
                     const float* inv_freq, int rot_dims, float eps, const int64_t* positions, void* kc, void* vc,
-                    const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf,
-                    hipStream_t stream);
+                    const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf, int layout,
+                    const float* q_scale, hipStream_t stream);
 void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
                         const float* bz, const float* bx, float* state, const int* cu_q, const int* start_pos,
                         const int* slots, int S, bool bf, hipStream_t stream);
@@ -98,15 +98,23 @@ void shift_state_update(torch::Tensor x, torch::Tensor w, double eps, torch::Ten
 
 void qk_prep(torch::Tensor q, torch::Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off, bool v_from_k,
              c10::optional<torch::Tensor> inv_freq, double eps, torch::Tensor positions, torch::Tensor kc,
-             torch::Tensor vc, torch::Tensor slot_mapping) {
+             torch::Tensor vc, torch::Tensor slot_mapping, int64_t layout, c10::optional<torch::Tensor> q_scale) {
   chk_act(q, "q"); chk_act(proj, "proj"); chk_act(kc, "k_cache"); chk_act(vc, "v_cache");
   TORCH_CHECK(q.scalar_type() == proj.scalar_type() && kc.scalar_type() == proj.scalar_type() &&
               vc.scalar_type() == proj.scalar_type(), "qk_prep: one dtype for proj, q and the cache");
   TORCH_CHECK(q.dim() == 3 && proj.dim() == 2 && kc.dim() == 4 && vc.dim() == 4, "qk_prep: ranks");
   const int64_t T = q.size(0), H = q.size(1), Dk = q.size(2);
-  const int64_t G = kc.size(1), BS = kc.size(2), Dv = vc.size(3), N = proj.size(1);
-  TORCH_CHECK(proj.size(0) == T && kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(2) == BS,
-              "qk_prep: shapes");
+  TORCH_CHECK(layout == 0 || layout == 1, "qk_prep: layout 0 (rows) or 1 (matrix-core kernels)");
+  // layout 1: values transposed per block, [nb, G, Dv, BS]; keys chunk-major in 32-entry chunks
+  const int64_t G = kc.size(1), BS = kc.size(2), Dv = vc.size(layout ? 2 : 3), N = proj.size(1);
+  TORCH_CHECK(proj.size(0) == T && kc.size(3) == Dk && vc.size(0) == kc.size(0) && vc.size(1) == G &&
+              vc.size(layout ? 3 : 2) == BS, "qk_prep: shapes");
+  TORCH_CHECK(layout == 0 || Dk % 32 == 0, "qk_prep: the matrix-core key layout needs dim % 32 == 0");
+  const float* qs = nullptr;
+  if (q_scale.has_value()) {
+    chk_f32(*q_scale, "q_scale", H);
+    qs = q_scale->data_ptr<float>();
+  }
   TORCH_CHECK(Dk >= 1 && Dk <= 256 && Dv >= 1 && Dv <= 256, "qk_prep: head sizes must be 1..256");
   TORCH_CHECK(q_off >= 0 && q_off + H * Dk <= N && k_off >= 0 && k_off + G * Dk <= N, "qk_prep: q / k columns");
   TORCH_CHECK(v_from_k ? Dv == Dk : (v_off >= 0 && v_off + G * Dv <= N), "qk_prep: v columns");
@@ -121,7 +129,7 @@ void qk_prep(torch::Tensor q, torch::Tensor proj, int64_t q_off, int64_t k_off, 
   chk_i64(positions, "positions", T); chk_i64(slot_mapping, "slot_mapping", T);
   launch_qk_prep(q.data_ptr(), proj.data_ptr(), N, q_off, k_off, v_off, v_from_k, fr, rot_dims, (float)eps,
                  positions.data_ptr<int64_t>(), kc.data_ptr(), vc.data_ptr(), slot_mapping.data_ptr<int64_t>(), T, H, G,
-                 Dk, Dv, BS, is_bf(q), cur());
+                 Dk, Dv, BS, is_bf(q), (int)layout, qs, cur());
 }
 
 void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor block_tables,

@@ -97,7 +97,7 @@ __global__ void __launch_bounds__(256) qk_prep_kernel(
     T* __restrict__ q, const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int v_from_k,
     const float* __restrict__ inv_freq, int rot_dims, float eps, const int64_t* __restrict__ positions,
     T* __restrict__ kc, T* __restrict__ vc, const int64_t* __restrict__ slot_mapping, int H, int G, int Dk, int Dv,
-    int BS) {
+    int BS, int layout, const float* __restrict__ q_scale) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float pos = (float)positions[t];
   const int64_t slot = slot_mapping[t];
@@ -126,18 +126,23 @@ __global__ void __launch_bounds__(256) qk_prep_kernel(
       val[j] = r;
       ss += r * r;
     }
-    const float k = inv_rms(rt::wave_sum(ss), Dk, eps);
-    T* dst = is_q ? q + ((size_t)t * H + u) * Dk : kc + (((size_t)blk * G + (u - H)) * BS + off) * Dk;
+    float k = inv_rms(rt::wave_sum(ss), Dk, eps);
+    if (is_q && q_scale) k *= q_scale[u];
+    // layout 1: the matrix-core attention kernels' cache (keys chunk-major per block, rt::kc_elem;
+    // values transposed [Dv][BS])
+    T* dst = is_q ? q + ((size_t)t * H + u) * Dk
+                  : kc + ((size_t)blk * G + (u - H)) * BS * Dk + (layout ? 0 : (size_t)off * Dk);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = lane + 64 * j;
-      if (d < Dk) DT<T>::store(dst + d, val[j] * k);
+      if (d < Dk) DT<T>::store(dst + ((!is_q && layout) ? rt::kc_elem(BS, off, d) : d), val[j] * k);
     }
     if (!is_q) {
       const int g = u - H;
       const T* vs = v_from_k ? src : row + v_off + g * Dv;
-      T* vd = vc + (((size_t)blk * G + g) * BS + off) * Dv;
-      for (int d = lane; d < Dv; d += 64) vd[d] = vs[d];
+      T* vd = vc + ((size_t)blk * G + g) * BS * Dv;
+      if (layout) for (int d = lane; d < Dv; d += 64) vd[(size_t)d * BS + off] = vs[d];
+      else for (int d = lane; d < Dv; d += 64) vd[(size_t)off * Dv + d] = vs[d];
     }
   }
 }
@@ -251,17 +256,17 @@ void launch_shift_state(const float* x, const float* w, float* state, const int*
 
 void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off, int v_off, bool v_from_k,
                     const float* inv_freq, int rot_dims, float eps, const int64_t* positions, void* kc, void* vc,
-                    const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf,
-                    hipStream_t stream) {
+                    const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf, int layout,
+                    const float* q_scale, hipStream_t stream) {
   if (T <= 0) return;
   if (bf)
     qk_prep_kernel<uint16_t><<<T, 256, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
                                                     v_from_k, inv_freq, rot_dims, eps, positions, (uint16_t*)kc,
-                                                    (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS);
+                                                    (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
   else
     qk_prep_kernel<float><<<T, 256, 0, stream>>>((float*)q, (const float*)proj, stride, q_off, k_off, v_off, v_from_k,
                                                  inv_freq, rot_dims, eps, positions, (float*)kc, (float*)vc,
-                                                 slot_mapping, H, G, Dk, Dv, BS);
+                                                 slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
 }
 
 void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,

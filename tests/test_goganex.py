@@ -546,3 +546,42 @@ def test_grouped_cache_slots_rollback_and_fork():
     kv.free_seq("a")
     kv.free_seq("c")
     assert kv.alloc.num_free == 8 and sorted(kv.state.free) == [0, 1]
+
+
+@GPU
+def test_layers_on_the_matrix_core_attention_kernels(tmp_path, monkeypatch):
+    """Shapes the framework's bf16 matrix-core attention kernels take (pages of 32, heads of 64 and
+    128, 1 to 4 query heads per key/value head): those layers keep their cache in the kernels'
+    layout, pass the sink on and move the head temperature into the queries. Prompts in portions,
+    a mixed batch and decode steps against the oracle and against the any-size kernel."""
+    from theroundtaible_amd import ops
+    from theroundtaible_amd.models.goganex import GoganexModel
+    if not ops.native_available():
+        pytest.skip("main extension not built")
+    cfg = make_config(width=64, vocab=80, loop=(1, 3, 2),
+                      layers=[att(4, 2, 64, ff=96, scale=0.2), par(2, 1, 128, 48, ff=0, scale=0.1),
+                              att(3, 1, 128, ff=0, scale=0.15), att(4, 4, 24, ff=32)])
+    P = make_checkpoint(tmp_path / "m", cfg, seed=12)
+    ta, tb = toks(150, cfg["vocab"], 12), toks(70, cfg["vocab"], 13)
+    wa, wb = O.forward(ta, P, cfg), O.forward(tb, P, cfg)
+    run = ("cuda:0", "bf16")
+    outs = []
+    for matrix in (True, False):
+        monkeypatch.setattr(GoganexModel, "matrix_attention", matrix)
+        e = engine_for(tmp_path / "m", run, block_size=32, tokens=1024)
+        assert e.kv.matrix == ([True, True, True, True, True, False] if matrix else [False] * 6)
+        ga = [e.step([("a", ta[:100], list(range(100)))])]
+        gb = []
+        o = e.step([("a", ta[100:101], [0]), ("b", tb[:45], list(range(45)))])
+        ga.append(o[:1]), gb.append(o[1:])
+        o = e.step([("a", ta[101:131], list(range(30))), ("b", tb[45:46], [0])])
+        ga.append(o[:30]), gb.append(o[30:])
+        for i in range(19):
+            o = e.step([("a", ta[131 + i:132 + i], [0]), ("b", tb[46 + i:47 + i], [0])])
+            ga.append(o[:1]), gb.append(o[1:])
+        gb.append(e.step([("b", tb[65:], list(range(5)))], end=["a", "b"]))
+        ga, gb = torch.cat(ga), torch.cat(gb)
+        close(ga, wa, run, f"a, matrix={matrix}")
+        close(gb, wb, run, f"b, matrix={matrix}")
+        outs.append((ga, gb))
+    assert float((outs[0][0] - outs[1][0]).abs().max()) < 0.25

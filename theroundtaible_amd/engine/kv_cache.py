@@ -296,7 +296,9 @@ class GroupedKVCache(StatefulPagedCache):
     Layer run ``l``: ``k[l]`` ``[num_blocks, kv_heads_l, block_size, dim_l]`` and ``v[l]``
     ``[num_blocks, kv_heads_l, block_size, vdim_l]``; token ``t`` of a sequence lives at
     ``block_tables[t // block_size]``, offset ``t % block_size``. ``shapes`` gives
-    ``(kv_heads, dim, vdim)`` per run.
+    ``(kv_heads, dim, vdim)`` per run. A run with ``matrix_layout`` keeps the layout of the
+    matrix-core attention kernels instead: ``v[l]`` ``[num_blocks, kv_heads_l, vdim_l, block_size]``
+    and each key block chunk-major (``ops/reference.py`` ``k_blocks``).
 
     States, fp32, one row per slot: ``shift[l]`` ``[n_slots, width]`` is the previous token's
     normed mixer input (token shift); ``rec[l]`` ``[n_slots, rec_width_l]`` the state of the
@@ -304,8 +306,11 @@ class GroupedKVCache(StatefulPagedCache):
     slot, so a reused slot needs no clearing."""
 
     def __init__(self, shapes, width: int, rec_widths, num_blocks: int, block_size: int, device,
-                 dtype=torch.bfloat16, n_slots: int = 16):
+                 dtype=torch.bfloat16, n_slots: int = 16, matrix_layout=None):
         self.n_layers = len(shapes)
+        # per run: the layout of the framework's matrix-core attention kernels (keys chunk-major
+        # per block, values transposed [.., vdim, block_size]) instead of plain rows
+        self.matrix = list(matrix_layout) if matrix_layout is not None else [False] * len(shapes)
         self.shapes = [tuple(int(x) for x in sh) for sh in shapes]
         self.n_kv_heads = max(sh[0] for sh in self.shapes)
         self.head_dim = max(max(sh[1], sh[2]) for sh in self.shapes)
@@ -313,7 +318,8 @@ class GroupedKVCache(StatefulPagedCache):
         self.device, self.dtype = device, dtype
         # zero-init: tail rows of a partial block are masked, never skipped, so they must be finite
         self.k = [torch.zeros(num_blocks, g, block_size, dk, dtype=dtype, device=device) for g, dk, _ in self.shapes]
-        self.v = [torch.zeros(num_blocks, g, block_size, dv, dtype=dtype, device=device) for g, _, dv in self.shapes]
+        self.v = [torch.zeros((num_blocks, g, dv, block_size) if mx else (num_blocks, g, block_size, dv), dtype=dtype,
+                              device=device) for (g, _, dv), mx in zip(self.shapes, self.matrix)]
         self.alloc = BlockAllocator(num_blocks)
         self.seqs = {}
         self.state = StateSlots(n_slots)

@@ -57,6 +57,7 @@ class _Rows:
 class GoganexModel:
     use_skinny = True          # decode steps run their linears on the skinny decode GEMM (A/B knob)
     fuse_adds = True           # residual adds ride in the next norm launch (A/B knob)
+    matrix_attention = True    # layers whose shapes fit run the framework's matrix-core attention kernels
     accepts_hidden = False
     stateful = True            # keeps a per-sequence running state beside the paged cache
 
@@ -111,11 +112,23 @@ class GoganexModel:
     def cache_shapes(self):
         return [(a.kv_heads, a.dim, a.vdim) for a in map(attention_of, self.cfg.layers)]
 
+    def matrix_layers(self, block_size: int, device, dtype):
+        """Per layer run: whether its attention runs on the framework's bf16 matrix-core kernels
+        (csrc/attention_prefill*.hip, attention_decode.hip, extended by the sink term): pages of
+        32 tokens, equal key and value size of 64 or 128, up to 16 query heads per key / value
+        head, the main extension built. Every other layer (and fp32) runs the family's own
+        any-size kernel on a cache of plain rows."""
+        from .. import ops
+        ok = (self.matrix_attention and torch.device(device).type == "cuda" and dtype == torch.bfloat16
+              and block_size == 32 and ops.native_available())
+        return [bool(ok and a.dim == a.vdim and a.dim in (64, 128) and a.group <= 16 and a.scale > 0)
+                for a in map(attention_of, self.cfg.layers)]
+
     def make_cache(self, num_blocks: int, block_size: int, device, dtype, n_slots: int):
         from ..engine.kv_cache import GroupedKVCache
         rec = [ls.mixer.right.width if isinstance(ls.mixer, ParallelSpec) else 0 for ls in self.cfg.layers]
         return GroupedKVCache(self.cache_shapes(), self.cfg.hidden, rec, num_blocks, block_size, device, dtype,
-                              n_slots=n_slots)
+                              n_slots=n_slots, matrix_layout=self.matrix_layers(block_size, device, dtype))
 
     def cache_bytes_per_block(self, block_size: int, dtype_bytes: int) -> int:
         return sum(g * (dk + dv) for g, dk, dv in self.cache_shapes()) * block_size * dtype_bytes
@@ -199,6 +212,8 @@ class GoganexModel:
     def _attend(self, proj, a, lw, l, positions, kv, meta, b, decode, v_off):
         """Queries / keys / values of ``proj`` -> cache -> attention output [T, heads * vdim]."""
         adt, T = self.dtype, proj.shape[0]
+        if kv.matrix[l]:
+            return self._attend_matrix(proj, a, lw, l, positions, kv, meta, b, decode, v_off)
         q = Hy.qk_prep(proj, a, 0, a.heads * a.dim, v_off, lw["inv_freq"], self.cfg.norm_eps, positions,
                        kv.k_layer(l), kv.v_layer(l), meta.slot_mapping, adt)
         splits = self.decode_splits(T, a.kv_heads) if decode else 1
@@ -206,6 +221,33 @@ class GoganexModel:
                                 lw.get("mix.temp") if a.head_temp else None, a.sink,
                                 tiles=self._tiles(meta, Hy.rows_per_tile(a.group), b) if proj.is_cuda else None,
                                 num_splits=splits, workspace=self._workspace(T, a, splits), out_dtype=adt)
+
+    def _attend_matrix(self, proj, a, lw, l, positions, kv, meta, b, decode, v_off):
+        """The same on the framework's matrix-core kernels: the cache in their layout, the head
+        temperature moved into the queries, the sink passed on."""
+        from .. import ops
+        T, dev = proj.shape[0], proj.device
+        kc, vc = kv.k_layer(l), kv.v_layer(l)
+        q = Hy.qk_prep(proj, a, 0, a.heads * a.dim, v_off, lw["inv_freq"], self.cfg.norm_eps, positions, kc, vc,
+                       meta.slot_mapping, self.dtype, matrix_layout=True,
+                       q_scale=lw.get("mix.temp") if a.head_temp else None)
+        if decode:
+            splits = ops.decode_splits(T, a.kv_heads)
+            key = ("matrix", T, a.heads, a.dim, splits)
+            ws = self._ws.get(key)
+            if ws is None:
+                ws = self._ws[key] = ops.DecodeWorkspace(T, a.heads, a.dim, splits, dev)
+            o = ops.paged_attention_decode(q, kc, vc, meta.block_tables, meta.ctx_lens, a.scale, splits, ws, sink=a.sink)
+        else:
+            rows = ops.native().prefill_rows_per_tile(a.group, a.dim)
+            cache = meta.latent_tiles if meta.latent_tiles is not None else {}
+            meta.latent_tiles = cache
+            tm = cache.get(("matrix", rows))
+            if tm is None:
+                cu, sp = meta.host_rows if meta.host_rows is not None else (b.cu_q.cpu(), b.start_pos.cpu())
+                tm = cache[("matrix", rows)] = ops.prefill_tile_map(cu, rows, sp).to(dev, non_blocking=True)
+            o = ops.prefill_attention(q, kc, vc, meta.block_tables, b.cu_q, b.start_pos, a.scale, tm, sink=a.sink)
+        return o.reshape(T, a.heads * a.vdim)
 
     def forward(self, ids: torch.Tensor, positions: torch.Tensor, kv, meta: AttnMeta,
                 hidden: Optional[torch.Tensor] = None, keep_layers: Optional[list] = None) -> torch.Tensor:

@@ -205,11 +205,12 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            block_tables: torch.Tensor, ctx_lens: torch.Tensor, scale: float,
                            num_splits: int = 1, workspace: Optional[DecodeWorkspace] = None,
                            out: Optional[torch.Tensor] = None, groups: Optional[torch.Tensor] = None,
-                           planned: bool = False) -> torch.Tensor:
+                           planned: bool = False, sink: float = 0.0) -> torch.Tensor:
     """``groups`` (optional, device ``[B, 3]`` int32 from :func:`decode_groups`): sequences whose
     block tables share leading blocks decode those keys once for the whole group. The result is
     identical to decoding every sequence alone (the fp32 oracle ignores ``groups``).
-    ``planned``: the workspace holds this step's :func:`attn_plan` for exactly these arguments."""
+    ``planned``: the workspace holds this step's :func:`attn_plan` for exactly these arguments.
+    ``sink``: a constant added to every softmax denominator as a key of score 0 without a value."""
     if _use_native(q):
         if out is None:
             out = torch.empty_like(q)
@@ -225,9 +226,9 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                                         int(num_splits), workspace.partial_o, workspace.partial_ml,
                                         workspace.counters, groups,
                                         workspace.slot_stride if groups is not None else 0, False,
-                                        plan, workspace.plan_stride if planned else 0)
+                                        plan, workspace.plan_stride if planned else 0, float(sink))
         return out
-    return ref.paged_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, scale)
+    return ref.paged_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, scale, sink=sink)
 
 
 def attn_plan(block_tables: torch.Tensor, ctx_lens: torch.Tensor, num_splits: int, workspace: DecodeWorkspace,
@@ -312,13 +313,16 @@ def prefill_split_plan(cu_q: torch.Tensor, rows_per_tile: int, start_pos, n_kv_h
 
 def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       cu_q: torch.Tensor, start_pos: torch.Tensor, scale: float,
-                      tile_map: Optional[torch.Tensor] = None, split=None) -> torch.Tensor:
+                      tile_map: Optional[torch.Tensor] = None, split=None, sink: float = 0.0) -> torch.Tensor:
     """``split``: a device-resident :func:`prefill_split_plan` ``(items, cmap, parts)`` — the
-    key-split launch + its combine; ``tile_map`` otherwise (whole tiles)."""
+    key-split launch + its combine; ``tile_map`` otherwise (whole tiles). ``sink``: a constant
+    added to every softmax denominator as a key of score 0 without a value (whole tiles only)."""
     if _use_native(q):
         nat = native()
         out = torch.empty_like(q)
         if split is not None:
+            if sink:
+                raise ValueError("prefill_attention: the key-split launch has no sink term")
             items, cmap, parts = split
             hkv, D = k_cache.shape[1], q.shape[2]
             part_o = torch.empty(parts * hkv * 8 * 32 * D, dtype=torch.float32, device=q.device)
@@ -329,9 +333,9 @@ def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         rows = nat.prefill_rows_per_tile(q.shape[1] // k_cache.shape[1], q.shape[2])
         if tile_map is None:
             tile_map = prefill_tile_map(cu_q.cpu(), rows, start_pos.cpu()).to(q.device)
-        nat.prefill_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, scale)
+        nat.prefill_attention(out, q, k_cache, v_cache, block_tables, cu_q, start_pos, tile_map, scale, float(sink))
         return out
-    return ref.prefill_attention(q, k_cache, v_cache, block_tables, cu_q.cpu(), start_pos.cpu(), scale)
+    return ref.prefill_attention(q, k_cache, v_cache, block_tables, cu_q.cpu(), start_pos.cpu(), scale, sink=sink)
 
 
 PRO_PLAIN, PRO_NORM, PRO_NORM_ADD = 0, 1, 2

@@ -100,19 +100,25 @@ def rotary_table(rot, device) -> Optional[torch.Tensor]:
 
 
 def qk_prep(proj, spec, q_off: int, k_off: int, v_off: int, inv_freq, eps, positions, k_cache, v_cache,
-            slot_mapping, out_dtype) -> torch.Tensor:
+            slot_mapping, out_dtype, matrix_layout: bool = False, q_scale=None) -> torch.Tensor:
     """``proj`` [T, N]: columns ``q_off ..`` hold the projected queries (heads x dim), ``k_off ..``
     the keys (kv_heads x dim), ``v_off ..`` the values (kv_heads x vdim; ignored when the values
     are the keys). Rotates the leading ``2 * len(inv_freq)`` entries of every query / key head
     (entry 2i with 2i + 1, angle = position * inv_freq[i], fp32), divides each head by its root
     mean square, writes keys and values to the paged cache at ``slot_mapping`` and returns the
-    queries [T, heads, dim]."""
+    queries [T, heads, dim]. ``matrix_layout`` (GPU): the cache of the framework's matrix-core
+    attention kernels — keys chunk-major per block, values transposed ``[nb, G, vdim, BS]``;
+    ``q_scale`` [heads] fp32 multiplies each query head (a per-head temperature moved into q)."""
     if _gpu(proj):
         T = proj.shape[0]
         q = torch.empty(T, spec.heads, spec.dim, dtype=out_dtype, device=proj.device)
         native().qk_prep(q, proj, int(q_off), int(k_off), int(v_off), bool(spec.value_from_key), inv_freq, float(eps),
-                         positions, k_cache, v_cache, slot_mapping)
+                         positions, k_cache, v_cache, slot_mapping, 1 if matrix_layout else 0, q_scale)
         return q
+    if matrix_layout:
+        raise ValueError("qk_prep: the matrix-core cache layout exists on the GPU only")
+    if q_scale is not None:
+        raise ValueError("qk_prep: q_scale is a GPU-path option (the CPU statement keeps the temperature in the scores)")
     return ref_qk_prep(proj, spec, q_off, k_off, v_off, inv_freq, eps, positions, k_cache, v_cache, slot_mapping,
                        out_dtype)
 

@@ -157,8 +157,18 @@ def _gather_kv(k_cache, v_cache, block_table, n):
     return k.float(), v.float()
 
 
+def _sink_softmax(s: torch.Tensor, sink: float) -> torch.Tensor:
+    """Softmax over the last axis with ``sink`` added to the denominator as exp(0) * sink."""
+    if not sink:
+        return torch.softmax(s, dim=-1)
+    m = s.max(-1, keepdim=True).values.clamp_min(0.0)
+    e = torch.exp(s - m)
+    return e / (e.sum(-1, keepdim=True) + sink * torch.exp(-m))
+
+
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                           block_tables: torch.Tensor, ctx_lens: torch.Tensor, scale: float) -> torch.Tensor:
+                           block_tables: torch.Tensor, ctx_lens: torch.Tensor, scale: float,
+                           sink: float = 0.0) -> torch.Tensor:
     B, Hq, D = q.shape
     Hkv = k_cache.shape[1]
     G = Hq // Hkv
@@ -168,7 +178,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)     # [n, Hkv, D]
         qb = q[b].float().reshape(Hkv, G, D)
         s = torch.einsum("hgd,nhd->hgn", qb, k) * scale
-        p = torch.softmax(s, dim=-1)
+        p = _sink_softmax(s, sink)
         o = torch.einsum("hgn,nhd->hgd", p, v)
         out[b] = o.reshape(Hq, D).to(q.dtype)
     return out
@@ -176,7 +186,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
 
 def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, cu_q: torch.Tensor, start_pos: torch.Tensor,
-                      scale: float) -> torch.Tensor:
+                      scale: float, sink: float = 0.0) -> torch.Tensor:
     """Varlen causal attention: sequence s has queries cu_q[s]:cu_q[s+1] at absolute positions
     start_pos[s] + i, attending to cached keys [0, start_pos[s] + i]."""
     T, Hq, D = q.shape
@@ -196,7 +206,7 @@ def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         kpos = torch.arange(n)[None, :]
         mask = (kpos <= qpos)[:, None, None, :]
         sc = sc.masked_fill(~mask, float("-inf"))
-        p = torch.softmax(sc, dim=-1)
+        p = _sink_softmax(sc, sink)
         o = torch.einsum("thgn,nhd->thgd", p, v)
         out[a:b] = o.reshape(b - a, Hq, D).to(q.dtype)
     return out
