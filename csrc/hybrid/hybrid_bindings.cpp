@@ -19,6 +19,11 @@ void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off,
 void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
                         const float* bz, const float* bx, float* state, const int* cu_q, const int* start_pos,
                         const int* slots, int S, bool bf, hipStream_t stream);
+int mingru_scan_chunk();
+void launch_mingru_chunked(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
+                           const float* bz, const float* bx, float* state, const int* cu_q, const int* start_pos,
+                           const int* slots, int S, const int* chunks, int n_chunks, const int* seq_chunk0, float* ws,
+                           bool bf, hipStream_t stream);
 void launch_dual_norm_add(float* x, const void* a, const float* wa, const void* b, const float* wb, int T, int W,
                           float eps, bool bf, hipStream_t stream);
 void launch_add_norm(void* out, float* x, const void* y, const float* w, int T, int W, float eps, bool out_bf,
@@ -175,7 +180,9 @@ void gqa_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kc, torch::
 }
 
 void mingru_scan(torch::Tensor out, torch::Tensor proj, int64_t z_off, int64_t x_off, int64_t g_off, torch::Tensor bz,
-                 torch::Tensor bx, torch::Tensor state, torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor slots) {
+                 torch::Tensor bx, torch::Tensor state, torch::Tensor cu_q, torch::Tensor start_pos, torch::Tensor slots,
+                 c10::optional<torch::Tensor> chunks, c10::optional<torch::Tensor> seq_chunk0,
+                 c10::optional<torch::Tensor> ws) {
   chk_act(out, "out"); chk_act(proj, "proj");
   TORCH_CHECK(out.dim() == 2 && proj.dim() == 2 && out.size(0) == proj.size(0) && out.scalar_type() == proj.scalar_type(),
               "mingru_scan: shapes");
@@ -184,6 +191,18 @@ void mingru_scan(torch::Tensor out, torch::Tensor proj, int64_t z_off, int64_t x
   chk_f32(bz, "bz", width); chk_f32(bx, "bx", width); chk_f32(state, "state");
   TORCH_CHECK(state.dim() == 2 && state.size(1) == width, "mingru_scan: state must be [slots, width]");
   chk_i32(cu_q, "cu_q", S + 1); chk_i32(start_pos, "start_pos", S); chk_i32(slots, "slots");
+  if (chunks.has_value()) {      // long spans: the three-launch chunked scan
+    TORCH_CHECK(seq_chunk0.has_value() && ws.has_value(), "mingru_scan: chunks need seq_chunk0 and the workspace");
+    chk_i32(*chunks, "chunks"); chk_i32(*seq_chunk0, "seq_chunk0", S + 1); chk_f32(*ws, "ws");
+    TORCH_CHECK(chunks->dim() == 2 && chunks->size(1) == 2, "mingru_scan: chunks [n, 2]");
+    const int64_t n = chunks->size(0);
+    TORCH_CHECK(ws->numel() >= 3 * n * width, "mingru_scan: workspace too small");
+    launch_mingru_chunked(out.data_ptr(), proj.data_ptr(), N, z_off, x_off, g_off, width, bz.data_ptr<float>(),
+                          bx.data_ptr<float>(), state.data_ptr<float>(), cu_q.data_ptr<int>(), start_pos.data_ptr<int>(),
+                          slots.data_ptr<int>(), S, chunks->data_ptr<int>(), n, seq_chunk0->data_ptr<int>(),
+                          ws->data_ptr<float>(), is_bf(proj), cur());
+    return;
+  }
   launch_mingru_scan(out.data_ptr(), proj.data_ptr(), N, z_off, x_off, g_off, width, bz.data_ptr<float>(),
                      bx.data_ptr<float>(), state.data_ptr<float>(), cu_q.data_ptr<int>(), start_pos.data_ptr<int>(),
                      slots.data_ptr<int>(), S, is_bf(proj), cur());
@@ -229,7 +248,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("qk_prep", &qk_prep);
   m.def("gqa_key_tile", [](int64_t Dk, int64_t Dv) { return gqa_key_tile((int)Dk, (int)Dv); });
   m.def("gqa_attention", &gqa_attention);
-  m.def("mingru_scan", &mingru_scan);
+  m.def("mingru_scan", &mingru_scan, py::arg("out"), py::arg("proj"), py::arg("z_off"), py::arg("x_off"), py::arg("g_off"),
+        py::arg("bz"), py::arg("bx"), py::arg("state"), py::arg("cu_q"), py::arg("start_pos"), py::arg("slots"),
+        py::arg("chunks") = py::none(), py::arg("seq_chunk0") = py::none(), py::arg("ws") = py::none());
+  m.def("mingru_scan_chunk", &mingru_scan_chunk);
   m.def("dual_norm_add", &dual_norm_add);
   m.def("add_norm", &add_norm);
   m.def("limited_glu", &limited_glu);

@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(1024) shift_state_kernel(const float* __restri
 // One wave per head unit: units 0 .. H - 1 are query heads, H .. H + G - 1 key heads (each also
 // writes its value head). A lane holds entries lane, lane + 64, ... of the head (at most 4).
 template <typename T>
-__global__ void __launch_bounds__(256) qk_prep_kernel(
+__global__ void __launch_bounds__(1024) qk_prep_kernel(
     T* __restrict__ q, const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int v_from_k,
     const float* __restrict__ inv_freq, int rot_dims, float eps, const int64_t* __restrict__ positions,
     T* __restrict__ kc, T* __restrict__ vc, const int64_t* __restrict__ slot_mapping, int H, int G, int Dk, int Dv,
@@ -171,6 +171,65 @@ __global__ void __launch_bounds__(256) mingru_scan_kernel(
   *st = S;
 }
 
+// The same recurrence for long spans, in three launches over chunks of kScanChunk rows: (1) every
+// chunk alone from S = 0: its decay product A and its end state B; (2) per sequence, chunk by
+// chunk: the state each chunk starts from (carry = A * carry + B), and the sequence's new state;
+// (3) every chunk again from its true start state, writing the outputs. chunks [n, 2] = (sequence,
+// first row), a sequence's chunks consecutive and in order; seq_chunk0 [S + 1] = first chunk of
+// each sequence.
+constexpr int kScanChunk = 64;
+
+template <typename T, int PASS>
+__global__ void __launch_bounds__(256) mingru_chunk_kernel(
+    T* __restrict__ out, const T* __restrict__ proj, int stride, int z_off, int x_off, int g_off, int width,
+    const float* __restrict__ bz, const float* __restrict__ bx, const int* __restrict__ cu_q,
+    const int* __restrict__ chunks, float* __restrict__ ws_a, float* __restrict__ ws_b,
+    const float* __restrict__ ws_in) {
+  const int k = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int s = chunks[2 * k], r0 = chunks[2 * k + 1];
+  const int r1 = min(r0 + kScanChunk, cu_q[s + 1]);
+  const float bzc = bz[c], bxc = bx[c];
+  float S = PASS == 1 ? 0.f : ws_in[(size_t)k * width + c];
+  float A = 1.f;
+  for (int r = r0; r < r1; ++r) {
+    const T* row = proj + (size_t)r * stride;
+    const float z = sigmoidf(DT<T>::load(row + z_off + c) + bzc);
+    const float u = DT<T>::load(row + x_off + c) + bxc;
+    const float cand = u >= 0.f ? u + 0.5f : sigmoidf(u);
+    S = (1.0f - z) * S + z * cand;
+    if (PASS == 1) {
+      A *= 1.0f - z;
+    } else {
+      const float g = DT<T>::load(row + g_off + c);
+      DT<T>::store(out + (size_t)r * width + c, S * (g * sigmoidf(g)));
+    }
+  }
+  if (PASS == 1) {
+    ws_a[(size_t)k * width + c] = A;
+    ws_b[(size_t)k * width + c] = S;
+  }
+}
+
+__global__ void __launch_bounds__(256) mingru_carry_kernel(const float* __restrict__ ws_a, const float* __restrict__ ws_b,
+                                                           float* __restrict__ ws_in, float* __restrict__ state,
+                                                           const int* __restrict__ seq_chunk0,
+                                                           const int* __restrict__ start_pos,
+                                                           const int* __restrict__ slots, int width) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int k0 = seq_chunk0[s], k1 = seq_chunk0[s + 1];
+  if (c >= width || k1 <= k0) return;
+  float* st = state + (size_t)slots[s] * width + c;
+  float S = start_pos[s] > 0 ? *st : 0.f;
+  for (int k = k0; k < k1; ++k) {
+    ws_in[(size_t)k * width + c] = S;
+    S = ws_a[(size_t)k * width + c] * S + ws_b[(size_t)k * width + c];
+  }
+  *st = S;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(1024) dual_norm_add_kernel(float* __restrict__ x, const T* __restrict__ a,
                                                              const float* __restrict__ wa, const T* __restrict__ b,
@@ -223,6 +282,26 @@ __global__ void __launch_bounds__(256) limited_glu_kernel(T* __restrict__ out, c
   DT<T>::store(out + i, g * sigmoidf(1.702f * g) * (u + 1.0f));
 }
 
+// bf16, F % 8 == 0: 16-byte loads and stores
+__global__ void __launch_bounds__(256) limited_glu8_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ gu,
+                                                           int64_t rows, int F, float limit) {
+  const int F8 = F >> 3;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * F8) return;
+  const int64_t r = i / F8;
+  const int c = (int)(i - r * F8) * 8;
+  const rt::short8 gv = *reinterpret_cast<const rt::short8*>(gu + r * 2 * F + c);
+  const rt::short8 uv = *reinterpret_cast<const rt::short8*>(gu + r * 2 * F + F + c);
+  rt::short8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float g = fminf(rt::bf2f((uint16_t)gv[j]), limit);
+    const float u = fminf(fmaxf(rt::bf2f((uint16_t)uv[j]), -limit), limit);
+    o[j] = (short)rt::f2bf(g * sigmoidf(1.702f * g) * (u + 1.0f));
+  }
+  *reinterpret_cast<rt::short8*>(out + r * F + c) = o;
+}
+
 int row_threads(int W) {
   int t = 64;
   while (t < 1024 && t * 4 < W) t *= 2;
@@ -259,12 +338,14 @@ void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off,
                     const int64_t* slot_mapping, int T, int H, int G, int Dk, int Dv, int BS, bool bf, int layout,
                     const float* q_scale, hipStream_t stream) {
   if (T <= 0) return;
+  // one wave per head unit, up to 16 waves a row: a decode step's few rows spread over whole workgroups
+  const int th = 64 * (H + G < 4 ? 4 : H + G > 16 ? 16 : H + G);
   if (bf)
-    qk_prep_kernel<uint16_t><<<T, 256, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
+    qk_prep_kernel<uint16_t><<<T, th, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
                                                     v_from_k, inv_freq, rot_dims, eps, positions, (uint16_t*)kc,
                                                     (uint16_t*)vc, slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
   else
-    qk_prep_kernel<float><<<T, 256, 0, stream>>>((float*)q, (const float*)proj, stride, q_off, k_off, v_off, v_from_k,
+    qk_prep_kernel<float><<<T, th, 0, stream>>>((float*)q, (const float*)proj, stride, q_off, k_off, v_off, v_from_k,
                                                  inv_freq, rot_dims, eps, positions, (float*)kc, (float*)vc,
                                                  slot_mapping, H, G, Dk, Dv, BS, layout, q_scale);
 }
@@ -281,6 +362,30 @@ void launch_mingru_scan(void* out, const void* proj, int stride, int z_off, int 
   else
     mingru_scan_kernel<float><<<grid, th, 0, stream>>>((float*)out, (const float*)proj, stride, z_off, x_off, g_off,
                                                        width, bz, bx, state, cu_q, start_pos, slots);
+}
+
+int mingru_scan_chunk() { return kScanChunk; }
+
+// ws: 3 * n_chunks * width floats
+void launch_mingru_chunked(void* out, const void* proj, int stride, int z_off, int x_off, int g_off, int width,
+                           const float* bz, const float* bx, float* state, const int* cu_q, const int* start_pos,
+                           const int* slots, int S, const int* chunks, int n_chunks, const int* seq_chunk0, float* ws,
+                           bool bf, hipStream_t stream) {
+  if (S <= 0 || width <= 0 || n_chunks <= 0) return;
+  const int th = width >= 256 ? 256 : 64;
+  const int cb = (width + th - 1) / th;
+  float *wa = ws, *wb = ws + (size_t)n_chunks * width, *wi = ws + 2 * (size_t)n_chunks * width;
+  dim3 gc(n_chunks, cb), gs(S, cb);
+#define RT_MG(TT)                                                                                                      \
+  do {                                                                                                                 \
+    mingru_chunk_kernel<TT, 1><<<gc, th, 0, stream>>>((TT*)out, (const TT*)proj, stride, z_off, x_off, g_off, width,  \
+                                                      bz, bx, cu_q, chunks, wa, wb, nullptr);                         \
+    mingru_carry_kernel<<<gs, th, 0, stream>>>(wa, wb, wi, state, seq_chunk0, start_pos, slots, width);               \
+    mingru_chunk_kernel<TT, 3><<<gc, th, 0, stream>>>((TT*)out, (const TT*)proj, stride, z_off, x_off, g_off, width,  \
+                                                      bz, bx, cu_q, chunks, nullptr, nullptr, wi);                    \
+  } while (0)
+  if (bf) RT_MG(uint16_t); else RT_MG(float);
+#undef RT_MG
 }
 
 void launch_dual_norm_add(float* x, const void* a, const float* wa, const void* b, const float* wb, int T, int W,
@@ -309,6 +414,10 @@ void launch_add_norm(void* out, float* x, const void* y, const float* w, int T, 
 void launch_limited_glu(void* out, const void* gu, int64_t rows, int F, float limit, bool bf, hipStream_t stream) {
   const int64_t n = rows * F;
   if (n <= 0) return;
+  if (bf && F % 8 == 0) {
+    limited_glu8_kernel<<<(int)((n / 8 + 255) / 256), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)gu, rows, F, limit);
+    return;
+  }
   const int blocks = (int)((n + 255) / 256);
   if (bf) limited_glu_kernel<uint16_t><<<blocks, 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)gu, rows, F, limit);
   else limited_glu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, rows, F, limit);

@@ -269,10 +269,11 @@ def test_prefill_against_token_by_token(tmp_path, run):
 
 
 @pytest.mark.parametrize("run", RUNS)
-@pytest.mark.parametrize("cuts", [[2, 2, 3, 1, 30, 2, 17, 1, 1, 5], [16, 16, 16, 16], [1, 63], [33, 31]])
+@pytest.mark.parametrize("cuts", [[2, 2, 3, 1, 30, 2, 17, 1, 1, 5], [16, 16, 16, 16], [1, 63], [33, 31], [131, 2, 70]])
 def test_portions(tmp_path, run, cuts):
     """Portions of several sizes, down to two tokens and one, cut inside and at page borders
-    (pages of 16): the shift state and the recurrence state carry over every cut."""
+    (pages of 16): the shift state and the recurrence state carry over every cut. The long portions
+    take the recurrence's chunked scan on the GPU."""
     cfg = make_config()
     P = make_checkpoint(tmp_path / "m", cfg, seed=4)
     e = engine_for(tmp_path / "m", run)

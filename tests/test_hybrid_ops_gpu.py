@@ -134,6 +134,14 @@ def test_mingru_scan(dt, width):
     got = Hy.mingru_scan(proj.to(DEV), 5, 5 + 2 * width, 5 + width, width, *gpu(bz, bx, st_g, cu, sp, slots), dt)
     torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
     torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-4, atol=1e-5)
+    # the chunked scan (spans of 130 rows = two chunks and a short one, beside single rows)
+    ch = Hy.scan_chunks(cu, DEV)
+    assert ch is not None and ch[0].shape[0] == 6 and ch[1].tolist() == [0, 1, 2, 3, 6]
+    st_g = state.clone().to(DEV)
+    got = Hy.mingru_scan(proj.to(DEV), 5, 5 + 2 * width, 5 + width, width, *gpu(bz, bx, st_g, cu, sp, slots), dt, chunks=ch)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dt))
+    torch.testing.assert_close(st_g.cpu(), st_c, rtol=1e-4, atol=1e-5)
+    assert Hy.scan_chunks(torch.tensor([0, 64, 65]), DEV) is None
 
 
 @pytest.mark.parametrize("dt", DTYPES)

@@ -193,6 +193,15 @@ class GoganexModel:
             t = cache[rows] = Hy.tile_map(cu, sp, rows).to(b.cu_q.device, non_blocking=True)
         return t
 
+    def _scan_chunks(self, meta: AttnMeta, b: _Rows):
+        """Work lists of the chunked recurrence scan for this batch (None: no long span)."""
+        cache = meta.latent_tiles if meta.latent_tiles is not None else {}
+        meta.latent_tiles = cache
+        if "scan" not in cache:
+            cu = meta.host_rows[0] if meta.host_rows is not None else b.cu_q.cpu()
+            cache["scan"] = Hy.scan_chunks(cu, b.cu_q.device)
+        return cache["scan"]
+
     def decode_splits(self, rows: int, kv_heads: int) -> int:
         """Key ranges per decoded row: about one workgroup per CU over rows x key/value heads."""
         if self.device.type != "cuda":
@@ -279,7 +288,8 @@ class GoganexModel:
                 o = self._attend(proj, a, lw, l, positions, kv, meta, b, decode, 0)
                 off = (a.heads + a.kv_heads) * a.dim
                 s = Hy.mingru_scan(proj, off, off + r.width, off + 2 * r.width, r.width, lw["mix.right.z.b"],
-                                   lw["mix.right.x.b"], kv.rec[l], b.cu_q, b.start_pos, b.slots, adt)
+                                   lw["mix.right.x.b"], kv.rec[l], b.cu_q, b.start_pos, b.slots, adt,
+                                   chunks=self._scan_chunks(meta, b) if proj.is_cuda and not decode else None)
                 Hy.dual_norm_add_(x, self._linear(o, src, "mix.left.o", skinny), lw["mix.left.out"],
                                   self._linear(s, src, "mix.right.o", skinny), lw["mix.right.out"], eps)
             else:

@@ -178,15 +178,41 @@ def gqa_attention(q, k_cache, v_cache, block_tables, cu_q, start_pos, scale: flo
 
 # ---- minGRU ---------------------------------------------------------------------------------------
 
+SCAN_CHUNK = 64          # rows per chunk of the chunked scan (csrc/hybrid/hybrid_ops.hip kScanChunk)
+
+
+def scan_chunks(cu_q: torch.Tensor, device=None):
+    """Work lists of the chunked scan from the host copy of ``cu_q``: (chunks [n, 2] int32 =
+    (sequence, first row), a sequence's chunks consecutive and in order; seq_chunk0 [S + 1] int32),
+    or None when no span is longer than one chunk (the one-launch scan is used then)."""
+    cq = cu_q.tolist()
+    if max((b - a for a, b in zip(cq, cq[1:])), default=0) <= SCAN_CHUNK:
+        return None
+    chunks, first = [], [0]
+    for s in range(len(cq) - 1):
+        chunks += [(s, r) for r in range(cq[s], cq[s + 1], SCAN_CHUNK)]
+        first.append(len(chunks))
+    return (torch.tensor(chunks, dtype=torch.int32).reshape(-1, 2).to(device, non_blocking=True),
+            torch.tensor(first, dtype=torch.int32).to(device, non_blocking=True))
+
+
 def mingru_scan(proj, z_off: int, x_off: int, g_off: int, width: int, bz, bx, state, cu_q, start_pos, slots,
-                out_dtype) -> torch.Tensor:
+                out_dtype, chunks=None) -> torch.Tensor:
     """``proj`` [T, N] holds the three projections of the recurrence at the given column offsets.
     z = sigmoid(p_z + bz); u = p_x + bx; c = u + 1/2 where u >= 0, sigmoid(u) below;
     S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, from ``state[slot]`` (zeros at position 0);
-    returns S_t * silu(p_g) [T, width] and leaves every span's last S in ``state``. fp32 inside."""
+    returns S_t * silu(p_g) [T, width] and leaves every span's last S in ``state``. fp32 inside.
+    ``chunks`` (GPU): :func:`scan_chunks` of this batch — spans are then scanned in chunks of
+    ``SCAN_CHUNK`` rows in parallel (chunk aggregates, a carry pass, the outputs) instead of row by
+    row; the results differ from the one-launch scan by rounding only."""
     if _gpu(proj):
         out = torch.empty(proj.shape[0], width, dtype=out_dtype, device=proj.device)
-        native().mingru_scan(out, proj, int(z_off), int(x_off), int(g_off), bz, bx, state, cu_q, start_pos, slots)
+        if chunks is not None:
+            ws = torch.empty(3 * chunks[0].shape[0] * width, dtype=torch.float32, device=proj.device)
+            native().mingru_scan(out, proj, int(z_off), int(x_off), int(g_off), bz, bx, state, cu_q, start_pos, slots,
+                                 chunks[0], chunks[1], ws)
+        else:
+            native().mingru_scan(out, proj, int(z_off), int(x_off), int(g_off), bz, bx, state, cu_q, start_pos, slots)
         return out
     return ref_mingru_scan(proj, z_off, x_off, g_off, width, bz, bx, state, cu_q, start_pos, slots, out_dtype)
 
