@@ -20,6 +20,7 @@ using rt::DT;
 
 RT_DEVICE float inv_rms(float ss, int n, float eps) { return 1.0f / sqrtf(ss / (float)n + eps); }
 RT_DEVICE float sigmoidf(float v) { return 1.0f / (1.0f + expf(-v)); }
+constexpr int kKeep = 4;    // entries per lane a two-pass row kernel keeps in registers (the rest are read again)
 
 // block-wide sum of two values at once
 RT_DEVICE void block_sum2(float& a, float& b, float* scratch) {
@@ -53,21 +54,42 @@ __global__ void __launch_bounds__(1024) shift_norm_kernel(
   const YT* yp = yr ? yr - W : nullptr;
   float* st = state + (size_t)slots[s] * W;
   float ss = 0.f, sp = 0.f;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+  float cv[kKeep], cu[kKeep];     // this row's and the row above's first entries per lane
+  int i = 0;
+  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
     const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
     ss += v * v;
+    float u = 0.f;
     if (!first) {
-      const float u = xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f);
+      u = xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f);
       sp += u * u;
     }
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+      if (j == i) {
+        cv[j] = v;
+        cu[j] = u;
+      }
   }
   block_sum2(ss, sp, scratch);
   const float kc = inv_rms(ss, W, eps), kp = inv_rms(sp, W, eps);
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+  i = 0;
+  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+    float v = 0.f, u = 0.f;
+    if (i < kKeep) {
+#pragma unroll
+      for (int j = 0; j < kKeep; ++j)
+        if (j == i) {
+          v = cv[j];
+          u = cu[j];
+        }
+    } else {
+      v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+      if (!first) u = xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f);
+    }
     const float h = v * kc * w[c];
     float hp;
-    if (!first) hp = (xp[c] + (yp ? DT<YT>::load(yp + c) : 0.f)) * kp * w[c];
+    if (!first) hp = u * kp * w[c];
     else hp = pos > 0 ? st[c] : 0.f;
     DT<OT>::store(out + (size_t)t * W + c, h + (hp - h) * mu[c]);
     if (yr) xs[(size_t)t * W + c] = v;
@@ -98,8 +120,16 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
     const float* __restrict__ inv_freq, int rot_dims, float eps, const int64_t* __restrict__ positions,
     T* __restrict__ kc, T* __restrict__ vc, const int64_t* __restrict__ slot_mapping, int H, int G, int Dk, int Dv,
     int BS, int layout, const float* __restrict__ q_scale) {
+  __shared__ float cs_tab[256];      // (cos, sin) of the row's angles, once for all its heads
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < (rot_dims >> 1); i += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    cs_tab[2 * i] = cs;
+    cs_tab[2 * i + 1] = sn;
+  }
+  __syncthreads();
   const int64_t slot = slot_mapping[t];
   const int64_t blk = slot / BS;
   const int off = (int)(slot - blk * BS);
@@ -118,8 +148,7 @@ __global__ void __launch_bounds__(1024) qk_prep_kernel(
         r = a;
         if (d < rot_dims) {
           const float b = DT<T>::load(src + (d ^ 1));
-          float sn, cs;
-          sincosf(pos * inv_freq[d >> 1], &sn, &cs);
+          const float cs = cs_tab[d & ~1], sn = cs_tab[d | 1];
           r = (d & 1) ? a * cs + b * sn : a * cs - b * sn;
         }
       }
@@ -258,13 +287,26 @@ __global__ void __launch_bounds__(1024) add_norm_kernel(OT* __restrict__ out, fl
   float* xr = x + (size_t)blockIdx.x * W;
   const YT* yr = y ? y + (size_t)blockIdx.x * W : nullptr;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+  float cv[kKeep];
+  int i = 0;
+  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
     const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
     ss += v * v;
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+      if (j == i) cv[j] = v;
   }
   const float k = inv_rms(rt::block_sum(ss, scratch), W, eps);
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    const float v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+  i = 0;
+  for (int c = threadIdx.x; c < W; c += blockDim.x, ++i) {
+    float v = 0.f;
+    if (i < kKeep) {
+#pragma unroll
+      for (int j = 0; j < kKeep; ++j)
+        if (j == i) v = cv[j];
+    } else {
+      v = xr[c] + (yr ? DT<YT>::load(yr + c) : 0.f);
+    }
     if (yr) xr[c] = v;
     DT<OT>::store(out + (size_t)blockIdx.x * W + c, v * k * w[c]);
   }
@@ -339,7 +381,7 @@ void launch_qk_prep(void* q, const void* proj, int stride, int q_off, int k_off,
                     const float* q_scale, hipStream_t stream) {
   if (T <= 0) return;
   // one wave per head unit, up to 16 waves a row: a decode step's few rows spread over whole workgroups
-  const int th = 64 * (H + G < 4 ? 4 : H + G > 16 ? 16 : H + G);
+  const int th = T > 64 ? 256 : 64 * (H + G < 4 ? 4 : H + G > 16 ? 16 : H + G);
   if (bf)
     qk_prep_kernel<uint16_t><<<T, th, 0, stream>>>((uint16_t*)q, (const uint16_t*)proj, stride, q_off, k_off, v_off,
                                                     v_from_k, inv_freq, rot_dims, eps, positions, (uint16_t*)kc,
