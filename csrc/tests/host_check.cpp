@@ -17,7 +17,7 @@ int launch_paged_decode(void* out, const void* q, const void* k_cache, const voi
                         const int* ctx_lens, float* part_o, float* part_ml, int* counters, int B, int Hq, int Hkv,
                         int D, int max_blocks, float scale, int num_splits, const int* groups, int slot_stride,
                         hipStream_t stream, int defer_combine, int* deferred, const int* plan = nullptr,
-                        int plan_stride = 0);
+                        int plan_stride = 0, float sink = 0.f);
 int launch_paging_guard(const int* block_tables, const int* ctx_lens, const int64_t* positions, const int64_t* slots,
                         int* err, int B, int max_blocks, int num_blocks, int BS, hipStream_t stream);
 int launch_decode_advance(int64_t* out, int64_t* ids, int64_t* positions, int* ctx_lens, int64_t* step,
