@@ -21,12 +21,13 @@ namespace {
 
 using rt::DT;
 
-constexpr int kPairs = 32;          // (row, head) pairs per workgroup
+constexpr int kPairs = 32;          // most (row, head) pairs per workgroup
 constexpr int kWaves = 4;
-constexpr int kPW = kPairs / kWaves;  // pairs per wave
 constexpr float kNeg = -1e30f;
 
-template <typename T, int DVL>      // DVL: value columns per lane (Dv <= 64 * DVL)
+// DVL: value columns per lane (Dv <= 64 * DVL); kPW: pairs per wave (8: varlen tiles of 32 pairs;
+// 2: the few pairs of a decode row, so no lane works on pairs that do not exist)
+template <typename T, int DVL, int kPW>
 __global__ void __launch_bounds__(256) gqa_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc,
     const int* __restrict__ block_tables, const int* __restrict__ cu_q, const int* __restrict__ start_pos,
@@ -49,8 +50,8 @@ __global__ void __launch_bounds__(256) gqa_attention_kernel(
   const int per = (ntile + S - 1) / S;
   const int t_lo = blockIdx.z * per, t_hi = min(ntile, t_lo + per);
 
-  float* qs = lds;                              // [kPairs][Dk]
-  float* ks = qs + kPairs * Dk;                 // [KT][Dk + 1]
+  float* qs = lds;                              // [kWaves * kPW][Dk]
+  float* ks = qs + kWaves * kPW * Dk;           // [KT][Dk + 1]
   float* vs = ks + KT * (Dk + 1);               // [KT][Dv]
   float* ps = vs + KT * Dv;                     // [kWaves][kPW][64]
   const int* bt = block_tables + (size_t)seq * max_blocks;
@@ -183,8 +184,8 @@ __global__ void __launch_bounds__(64) gqa_combine_kernel(T* __restrict__ out, co
   }
 }
 
-size_t lds_bytes(int Dk, int Dv, int KT) {
-  return sizeof(float) * ((size_t)kPairs * Dk + (size_t)KT * (Dk + 1) + (size_t)KT * Dv + kWaves * kPW * 64);
+size_t lds_bytes(int Dk, int Dv, int KT, int pairs = kPairs) {
+  return sizeof(float) * ((size_t)pairs * Dk + (size_t)KT * (Dk + 1) + (size_t)KT * Dv + pairs * 64);
 }
 
 }  // namespace
@@ -206,12 +207,18 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
   const int group = H / G;
   const int hchunks = (group + kPairs - 1) / kPairs;
   if (rows * (group < kPairs ? group : kPairs) > kPairs) return -2;
-  const size_t shm = lds_bytes(Dk, Dv, KT);
+  // pairs per wave: 2 when a workgroup has at most 8 pairs (decode rows of up to 8 heads per group)
+  const int pw = rows * (group < kPairs ? group : kPairs) <= 2 * kWaves ? 2 : 8;
+  const size_t shm = lds_bytes(Dk, Dv, KT, kWaves * pw);
   dim3 grid(n_tiles, G * hchunks, num_splits);
   const int dvl = Dv <= 64 ? 1 : Dv <= 128 ? 2 : 4;
 #define RT_GQA(TT, DVL)                                                                                              \
   do {                                                                                                               \
-    auto kern = gqa_attention_kernel<TT, DVL>;                                                                       \
+    if (pw == 2) RT_GQA2(TT, DVL, 2); else RT_GQA2(TT, DVL, 8);                                                      \
+  } while (0)
+#define RT_GQA2(TT, DVL, PW)                                                                                         \
+  do {                                                                                                               \
+    auto kern = gqa_attention_kernel<TT, DVL, PW>;                                                                    \
     if (shm > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,        \
                                                (int)shm) != hipSuccess)                                              \
       return -3;                                                                                                     \
@@ -225,6 +232,7 @@ int launch_gqa_attention(void* out, const void* q, const void* kc, const void* v
     if (dvl == 1) RT_GQA(float, 1); else if (dvl == 2) RT_GQA(float, 2); else RT_GQA(float, 4);
   }
 #undef RT_GQA
+#undef RT_GQA2
   if (num_splits > 1) {
     if (bf) gqa_combine_kernel<uint16_t><<<T * H, 64, 0, stream>>>((uint16_t*)out, part_o, part_ml, num_splits, Dv, sink);
     else gqa_combine_kernel<float><<<T * H, 64, 0, stream>>>((float*)out, part_o, part_ml, num_splits, Dv, sink);
